@@ -17,7 +17,7 @@ printed and flushed.  Nothing is sampled.
 The cache pool is made for ``--max-tokens`` tokens (every live request's count rounded up to a
 multiple of 64, or of the page size when that is larger), in pages of ``--kv-block-size`` tokens
 (default 16); ``--num-kv-blocks`` gives the number of pages outright and ``--max-live`` the most
-requests live at a time (default 8).  A trace may carry the same geometry itself, as a line before
+requests live at a time (default 4).  A trace may carry the same geometry itself, as a line before
 its first step, which then wins over the options:
 
     {"geometry": {"kv_block_size": 8, "num_kv_blocks": 40, "max_live": 4}}
@@ -58,7 +58,7 @@ def main(argv=None) -> int:
     ap.add_argument("--kv-block-size", type=int, default=16, help="tokens a page of the cache holds (default 16)")
     ap.add_argument("--num-kv-blocks", type=int, default=0,
                     help="pages of the cache pool (default: what --max-tokens needs)")
-    ap.add_argument("--max-live", type=int, default=8, help="most requests live at a time (default 8)")
+    ap.add_argument("--max-live", type=int, default=4, help="most requests live at a time (default 4)")
     args = ap.parse_args(argv)
     if args.max_tokens <= 0:
         ap.error("--max-tokens must be positive")

@@ -194,3 +194,89 @@ def read_config_json(path: str) -> Dict[str, Any]:
             return json.load(f)
         except json.JSONDecodeError as e:
             raise ConfigError(f"{path} is not valid JSON: {e}") from e
+
+
+@dataclass(frozen=True)
+class DedelornConfig(ModelConfig):
+    """The Dedelorn design's config.json: ``width``, ``vocab``, ``norm.eps`` and a list ``layers`` whose entries
+    each name a mixer by ``type`` ("delta": a gated delta rule; "latent_attention": windowed attention over cached
+    latents) with its sizes under ``mixer`` and a feed-forward under ``mlp`` (``kind`` "dense" or "moe", or null for
+    none).  Every size and constant of a model is read from here; the shared keys of ``ModelConfig`` that the
+    format does not have keep their neutral values (no end-of-sequence token, no position limit)."""
+
+    layers: Tuple[Any, ...] = ()
+    norm_eps: float = 1e-6
+
+    MIXER_KEYS = {"delta": ("heads", "kv_heads", "dim", "vdim", "conv"),
+                  "latent_attention": ("heads", "dim", "rot_dim", "vdim", "kv_rank", "scale", "rot")}
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "DedelornConfig":
+        missing = [k for k in ("width", "vocab", "layers", "norm") if k not in d]
+        if missing:
+            raise ConfigError("config.json lacks required key(s): " + ", ".join(missing))
+        if not isinstance(d["layers"], (list, tuple)) or not d["layers"]:
+            raise ConfigError("config.json: 'layers' must be a non-empty list")
+        if not isinstance(d["norm"], Mapping) or "eps" not in d["norm"]:
+            raise ConfigError("config.json: 'norm' must give 'eps'")
+        eos = d.get("eos_token_id")
+        cfg = cls(architectures=(str(d.get("architecture", "Dedelorn")),), model_type="dedelorn",
+                  torch_dtype=str(d.get("torch_dtype") or "bfloat16"), hidden_size=_as_int(d, "width"),
+                  vocab_size=_as_int(d, "vocab"), num_hidden_layers=len(d["layers"]),
+                  eos_token_ids=() if eos is None else tuple(int(e) for e in (eos if isinstance(eos, (list, tuple)) else [eos])),
+                  layers=tuple(json.loads(json.dumps(layer)) for layer in d["layers"]), norm_eps=float(d["norm"]["eps"]))
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.hidden_size <= 0 or self.vocab_size <= 0:
+            raise ConfigError("config.json: 'width' and 'vocab' must be positive")
+        if not (self.norm_eps > 0):
+            raise ConfigError(f"config.json: norm.eps must be positive, got {self.norm_eps}")
+        for i, layer in enumerate(self.layers):
+            kind = layer.get("type") if isinstance(layer, Mapping) else None
+            if kind not in self.MIXER_KEYS:
+                raise ConfigError(f"config.json: layer {i} has type {kind!r}; known: {', '.join(sorted(self.MIXER_KEYS))}")
+            m = layer.get("mixer")
+            lacking = [k for k in self.MIXER_KEYS[kind] if not isinstance(m, Mapping) or k not in m]
+            if lacking:
+                raise ConfigError(f"config.json: layer {i} ({kind}) lacks mixer key(s): " + ", ".join(lacking))
+            if kind == "delta":
+                if m["heads"] % m["kv_heads"]:
+                    raise ConfigError(f"config.json: layer {i}: heads {m['heads']} is not a multiple of kv_heads {m['kv_heads']}")
+            else:
+                if m["rot"].get("dims") != m["rot_dim"] or m["rot_dim"] % 2 or not m["rot"].get("base", 0) > 0:
+                    raise ConfigError(f"config.json: layer {i}: rot.dims must equal rot_dim and be even, rot.base positive")
+                if m.get("mask") is not None and not int(m["mask"].get("size", 0)) > 0:
+                    raise ConfigError(f"config.json: layer {i}: mask.size must be positive")
+                src = m.get("kv_from")
+                if src is not None:
+                    ok = isinstance(src, int) and 0 <= src < i and self.layers[src].get("type") == "latent_attention" \
+                        and self.layers[src]["mixer"].get("kv_from") is None
+                    if ok:
+                        o = self.layers[src]["mixer"]
+                        ok = (o["kv_rank"], o["rot_dim"], o["rot"]) == (m["kv_rank"], m["rot_dim"], m["rot"])
+                    if not ok:
+                        raise ConfigError(f"config.json: layer {i}: kv_from must name an earlier latent_attention layer with "
+                                          "a projection of its own and the same kv_rank, rot_dim and rot")
+            mlp = layer.get("mlp")
+            if mlp is None:
+                continue
+            if mlp.get("kind") == "dense":
+                if not int(mlp.get("ff", 0)) > 0:
+                    raise ConfigError(f"config.json: layer {i}: a dense mlp needs a positive 'ff'")
+            elif mlp.get("kind") == "moe":
+                r = mlp.get("router") or {}
+                if not int((mlp.get("expert") or {}).get("ff", 0)) > 0 or not (0 < int(r.get("top", 0)) <= int(r.get("experts", 0))):
+                    raise ConfigError(f"config.json: layer {i}: a moe mlp needs expert.ff, router.experts and router.top "
+                                      "(at most the experts)")
+            else:
+                raise ConfigError(f"config.json: layer {i}: mlp.kind {mlp.get('kind')!r} is neither 'dense' nor 'moe'")
+
+    def to_dict(self) -> Dict[str, Any]:
+        d = {"architecture": self.architectures[0] if self.architectures else "Dedelorn",
+             "layers": json.loads(json.dumps(list(self.layers))), "norm": {"eps": self.norm_eps},
+             "vocab": self.vocab_size, "width": self.hidden_size}
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids)
+        return d

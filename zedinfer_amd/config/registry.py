@@ -42,7 +42,9 @@ def registered_architectures() -> Tuple[str, ...]:
 
 
 def find_architecture(config_dict: Mapping[str, Any]) -> Architecture:
-    archs = config_dict.get("architectures") or []
+    archs = list(config_dict.get("architectures") or [])
+    if isinstance(config_dict.get("architecture"), str):      # some formats name their one architecture so
+        archs.insert(0, config_dict["architecture"])
     for a in archs:
         if a in _ARCHITECTURES:
             return _ARCHITECTURES[a]

@@ -201,3 +201,38 @@ extern "C" int zi_swiglu(void* out, int out_dt, const void* gate, const void* up
     }
     return zi_check_launch("swiglu");
 }
+
+// out = act(gate) * up, element by element, float32 arithmetic: the gated feed-forward's middle for activations
+// other than the one the SwiGLU kernels above carry.  act: 0 SiLU, 1 GELU in its tanh form
+// 0.5 z (1 + tanh(sqrt(2 / pi) (z + 0.044715 z^3))), 2 GELU with the error function.
+#define ZI_ACT_SILU 0
+#define ZI_ACT_GELU_TANH 1
+#define ZI_ACT_GELU_ERF 2
+
+__device__ __forceinline__ float zi_activation(float z, int act) {
+    if (act == ZI_ACT_GELU_TANH) return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
+    if (act == ZI_ACT_GELU_ERF) return 0.5f * z * (1.f + erff(z * 0.70710678118654752440f));
+    return z / (1.f + expf(-z));
+}
+
+template <typename T, typename TO>
+__global__ void gated_act_kernel(TO* __restrict__ out, int64_t ldo, const T* __restrict__ gate, const T* __restrict__ up,
+                                 int64_t ld_gate, int64_t ld_up, int n, int inter, int act) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)n * inter) return;
+    const int64_t r = i / inter, c = i % inter;
+    zi_store(out + r * ldo + c, zi_activation(zi_load(gate + r * ld_gate + c), act) * zi_load(up + r * ld_up + c));
+}
+
+extern "C" int zi_gated_act(void* out, int out_dt, int64_t ldo, const void* gate, const void* up, int dt, int64_t ld_gate,
+                            int64_t ld_up, int n, int inter, int act, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && inter > 0 && ldo >= inter && ld_gate >= inter && ld_up >= inter, "gated_act: bad sizes");
+    ZI_REQUIRE(act >= ZI_ACT_SILU && act <= ZI_ACT_GELU_ERF, "gated_act: unknown activation %d", act);
+    if (n == 0) return 0;
+    const int64_t total = (int64_t)n * inter;
+    ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(out_dt, TO, {
+        gated_act_kernel<T, TO><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(
+            (TO*)out, ldo, (const T*)gate, (const T*)up, ld_gate, ld_up, n, inter, act);
+    }));
+    return zi_check_launch("gated_act");
+}

@@ -87,6 +87,55 @@ int zi_rope(void* out, const void* in, int dt, int n, int64_t ld_in, int64_t ld_
     inv_freq, int nh, int d, int rot, hipStream_t stream);
 // rope_kv.hip
 int zi_rope_table(float* out, const int32_t* pos, const float* inv_freq, int n, int half, hipStream_t stream);
+// elementwise.hip
+int zi_gated_act(void* out, int out_dt, int64_t ldo, const void* gate, const void* up, int dt, int64_t ld_gate, int64_t
+    ld_up, int n, int inter, int act, hipStream_t stream);
+// latent.hip
+int zi_rope_pairs(void* x, int dt, int64_t ld, const float* table, int n, int heads, int d, int rot, hipStream_t
+    stream);
+// latent.hip
+int zi_latent_store(const float* dkv, int dt, int64_t ld, int n, const void* norm_w, int w_dt, float eps, const float*
+    table, const int32_t* slots, void* c_cache, void* kr_cache, int64_t cache_slots, int rank, int rot, hipStream_t
+    stream);
+// latent.hip
+int zi_latent_query(float* qa, const void* q, int dt, int64_t ldq, const void* w_uk, int w_dt, const float* table, int
+    n, int heads, int dim, int rank, int rot, hipStream_t stream);
+// latent.hip
+int zi_latent_attention(float* out, const float* qa, const void* c_cache, const void* kr_cache, int dt, int n_idx, const
+    int32_t* tok_index, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables, int max_pages, int
+    num_pages, int heads, int rank, int rot, int page_size, int window, float scale, hipStream_t stream);
+// latent.hip
+int zi_latent_value(void* out, int out_dt, int64_t ldo, const float* o, const void* w_uv, int w_dt, int n, int heads,
+    int vdim, int rank, hipStream_t stream);
+// delta.hip
+int zi_delta_prepare(float* qk, float* v, float* beta_g, const float* proj, int64_t ld, int n, const void* conv_w, const
+    void* a_log, const void* dt_bias, int w_dt, const float* state, int64_t state_stride, int64_t conv_off, const
+    int32_t* tok_seq, const int32_t* entry_start, const int32_t* entry_slot, int heads, int kvh, int dim, int vdim, int
+    taps, hipStream_t stream);
+// delta.hip
+int zi_delta_conv_state(float* state, int64_t state_stride, int64_t conv_off, const float* proj, int64_t ld, const
+    int32_t* entry_start, const int32_t* entry_len, const int32_t* entry_slot, int entries, int channels, int taps,
+    hipStream_t stream);
+// delta.hip
+int zi_delta_rule(float* out, const float* qk, const float* v, const float* beta_g, float* state, int64_t
+    state_stride, const int32_t* entry_start, const int32_t* entry_len, const int32_t* entry_slot, int entries, int
+    heads, int kvh, int dim, int vdim, hipStream_t stream);
+// delta.hip
+int zi_gated_rmsnorm(void* out, int out_dt, const float* o, const void* w, int w_dt, const float* gate, int64_t
+    ld_gate, int n, int heads, int vdim, float eps, hipStream_t stream);
+// moe.hip
+int zi_moe_route(int32_t* idx, float* wt, const float* z, const float* correction, int n, int experts, int top, float
+    scale, hipStream_t stream);
+// moe.hip
+int zi_moe_group(int32_t* plan, int32_t* order, int32_t* place_of, const int32_t* idx, int pairs, int experts, int
+    tile_rows, hipStream_t stream);
+// moe.hip
+int zi_moe_linear(void* out, int out_dt, int64_t ldo, const void* x, int x_dt, int64_t ldx, const void* w, int w_dt,
+    const int32_t* plan, const int32_t* source, int source_div, int max_tiles, int tile_rows, int N, int K, int act,
+    hipStream_t stream);
+// moe.hip
+int zi_moe_combine(float* out, const float* y, const float* wt, const int32_t* place_of, int n, int top, int hidden,
+    hipStream_t stream);
 // sampling.hip
 int zi_argmax(int32_t* out_idx, float* out_val, const void* logits, int dt, int rows, int vocab, int64_t ld, float*
     workspace, int64_t workspace_floats, hipStream_t stream);
@@ -119,5 +168,19 @@ int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int ro
     X(zi_rope_kv_store_split) \
     X(zi_rope) \
     X(zi_rope_table) \
+    X(zi_gated_act) \
+    X(zi_rope_pairs) \
+    X(zi_latent_store) \
+    X(zi_latent_query) \
+    X(zi_latent_attention) \
+    X(zi_latent_value) \
+    X(zi_delta_prepare) \
+    X(zi_delta_conv_state) \
+    X(zi_delta_rule) \
+    X(zi_gated_rmsnorm) \
+    X(zi_moe_route) \
+    X(zi_moe_group) \
+    X(zi_moe_linear) \
+    X(zi_moe_combine) \
     X(zi_argmax) \
     X(zi_sample)

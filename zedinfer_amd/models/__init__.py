@@ -1,4 +1,4 @@
-from . import qwen2  # noqa: F401  (registers the architecture)
+from . import dedelorn, qwen2  # noqa: F401  (register the architectures)
 from .model import DecoderModel, expected_weights
 
-__all__ = ["DecoderModel", "expected_weights", "qwen2"]
+__all__ = ["DecoderModel", "expected_weights", "dedelorn", "qwen2"]

@@ -96,8 +96,16 @@ class DecoderModel:
                 continue
             if st.cache in out and out[st.cache].tensors != req.tensors:
                 raise ValueError(f"cache {st.cache} is shared by layers that keep different tensors in a page")
-            if st.writes_cache or st.cache not in out:
+            if st.cache not in out:
                 out[st.cache] = req
+            else:
+                # the cache keeps what every layer that reads it can still see: all keys when one of them sees
+                # all, else the widest of their windows (each layer's kernels apply its own)
+                had = out[st.cache]
+                if "full" in (had.kind, req.kind):
+                    out[st.cache] = KVCacheRequest("full", 0, req.tensors)
+                else:
+                    out[st.cache] = KVCacheRequest(req.kind, max(had.window, req.window), req.tensors)
         return out
 
     def state_requests(self) -> Dict[int, StateRequest]:

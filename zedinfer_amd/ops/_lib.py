@@ -65,6 +65,20 @@ _PROTOTYPES = {
     "zi_gemm_skinny_supported": [I, I, I, L, L],
     "zi_argmax": [P, P, P, I, I, I, L, P, L, P],
     "zi_sample": [P, P, L, P, I, I, P, P, P, P, P, P, P, I, P],
+    "zi_gated_act": [P, I, L, P, P, I, L, L, I, I, I, P],
+    "zi_rope_pairs": [P, I, L, P, I, I, I, I, P],
+    "zi_latent_store": [P, I, L, I, P, I, F, P, P, P, P, L, I, I, P],
+    "zi_latent_query": [P, P, I, L, P, I, P, I, I, I, I, I, P],
+    "zi_latent_attention": [P, P, P, P, I, I, P, P, P, P, I, I, I, I, I, I, I, F, P],
+    "zi_latent_value": [P, I, L, P, P, I, I, I, I, I, P],
+    "zi_delta_prepare": [P, P, P, P, L, I, P, P, P, I, P, L, L, P, P, P, I, I, I, I, I, P],
+    "zi_delta_conv_state": [P, L, L, P, L, P, P, P, I, I, I, P],
+    "zi_delta_rule": [P, P, P, P, P, L, P, P, P, I, I, I, I, I, P],
+    "zi_gated_rmsnorm": [P, I, P, P, I, P, L, I, I, I, F, P],
+    "zi_moe_route": [P, P, P, P, I, I, I, F, P],
+    "zi_moe_group": [P, P, P, P, I, I, I, P],
+    "zi_moe_linear": [P, I, L, P, I, L, P, I, P, P, I, I, I, I, I, I, P],
+    "zi_moe_combine": [P, P, P, P, I, I, I, P],
     "zi_tape_record": [P, c_char_p, P, I],
     "zi_tape_record_many": [P, c_char_p, P, P, I],
     "zi_tape_run": [P, P],

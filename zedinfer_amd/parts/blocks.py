@@ -5,6 +5,8 @@ from typing import Optional
 
 import torch
 
+from .. import ops
+
 from .base import Block, LayerMemory, Runtime, register_block
 
 
@@ -31,3 +33,45 @@ class PreNormBlock(Block):
         a = self.mixer.forward(x, batch, memory)
         y = self.norm_post.add_forward(resid, a)
         return self.feed_forward.forward(y)
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """n = norm(h); h += mixer(n) + feed_forward(n): one norm, and both sublayers read its output.  The two
+    additions are handed on as a stack of float32 terms that the next norm adds into the float32 residual stream,
+    mixer first.  A sublayer that takes ``out=`` (``writes_into``) writes its term in place; any other result is
+    brought into the stack (a stack of partial sums added up, a bfloat16 result widened).  The feed-forward may be
+    the kind "none"."""
+
+    graph_safe = True
+    tape_safe = True
+
+    norm_names = ("input",)
+
+    def __init__(self, norms, mixer, feed_forward, rt: Runtime):
+        self.norm_in = norms["input"]
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.has_ff = getattr(feed_forward, "kind", "") != "none"
+        self.rt = rt
+        # a term that has to be copied into the stack is copied by a torch operator, which a tape does not hold
+        self.tape_safe = all(getattr(p, "writes_into", False) for p in ((mixer, feed_forward) if self.has_ff else (mixer,)))
+
+    def _term(self, slot: torch.Tensor, part, *args):
+        if getattr(part, "writes_into", False):
+            part.forward(*args, out=slot)
+            return
+        y = part.forward(*args)
+        if y.dim() == 3:
+            ops.reduce_sums(y, out=slot)
+        else:
+            slot.copy_(y)
+
+    def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], batch, memory: LayerMemory):
+        x = self.norm_in.add_forward(resid, delta) if delta is not None else self.norm_in.forward(resid)
+        n, H = resid.shape
+        terms = self.rt.buffer("parallel_terms", (2 if self.has_ff else 1, n, H), torch.float32)
+        self._term(terms[0], self.mixer, x, batch, memory)
+        if self.has_ff:
+            self._term(terms[1], self.feed_forward, x)
+        return terms

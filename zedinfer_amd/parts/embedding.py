@@ -14,23 +14,32 @@ from .base import Part, Runtime, register_embedding, register_head
 @register_embedding("token")
 class TokenEmbedding(Part):
     """h[i,:] = table[ids[i],:], unscaled, widened into the float32 residual stream
-    (reference: src/frontend/models/transformer_forward.cpp:54-60).  params: vocab_size, hidden_size."""
+    (reference: src/frontend/models/transformer_forward.cpp:54-60).  With ``norm_eps`` the rows are then RMS-normed
+    in place, in float32, with the gain ``norm`` [hidden_size].  params: vocab_size, hidden_size, norm_eps (None)."""
 
     graph_safe = True
     tape_safe = True
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
-        return {"weight": WeightSpec((int(spec.params["vocab_size"]), int(spec.params["hidden_size"])))}
+        w = {"weight": WeightSpec((int(spec.params["vocab_size"]), int(spec.params["hidden_size"])))}
+        if spec.params.get("norm_eps") is not None:
+            w["norm"] = WeightSpec((int(spec.params["hidden_size"]),), init="ones")
+        return w
 
     def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
         super().__init__(spec, weights, rt)
         self.weight = weights["weight"]
         self.vocab, self.hidden = self.weight.shape
+        self.norm_eps = spec.params.get("norm_eps")
+        self.norm = weights["norm"] if self.norm_eps is not None else None
 
     def forward(self, ids: torch.Tensor) -> torch.Tensor:
         out = self.rt.buffer("resid", (ids.numel(), self.hidden), torch.float32)
-        return ops.embedding(ids, self.weight, out=out)
+        ops.embedding(ids, self.weight, out=out)
+        if self.norm is not None:
+            ops.rms_norm(out, self.norm, float(self.norm_eps), out=out)      # a thread rewrites what it read itself
+        return out
 
 
 @register_head("linear")

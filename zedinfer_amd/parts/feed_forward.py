@@ -158,3 +158,131 @@ class SwiGLU(FeedForward):
             return ops.linear_sums(act, self.down, out=self.rt.buffer("ffn_out_sums", (S, n, self.hidden), torch.float32))
         out = self.rt.buffer("ffn_out", (n, self.hidden))
         return ops.linear(act, self.down, out=out)
+
+
+@register_feed_forward("none")
+class NoFeedForward(FeedForward):
+    """A layer without a feed-forward: block arrangements that know the kind leave the term out."""
+
+    graph_safe = True
+    tape_safe = True
+    writes_into = True
+
+    def forward(self, x: torch.Tensor, out=None):
+        return None
+
+
+@register_feed_forward("gated_mlp")
+class GatedMLP(FeedForward):
+    """down(act(gate(x)) * up(x)), no biases, with the activation as a parameter: "silu", "gelu_tanh"
+    (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3)))) or "gelu_erf".  gate and up are stacked into one [2I, H]
+    matrix at load (one product); the activation and the product of the halves are one kernel in float32
+    arithmetic.  With ``out=`` the result goes there (float32 for a float32 residual term).
+    params: hidden_size, intermediate_size, activation."""
+
+    graph_safe = True
+    tape_safe = True
+    writes_into = True
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        H, I = int(spec.params["hidden_size"]), int(spec.params["intermediate_size"])
+        return {"gate": WeightSpec((I, H)), "up": WeightSpec((I, H)), "down": WeightSpec((H, I))}
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        self.hidden = int(spec.params["hidden_size"])
+        self.inter = int(spec.params["intermediate_size"])
+        self.activation = str(spec.params.get("activation", "silu"))
+        if self.activation not in ("silu", "gelu_tanh", "gelu_erf"):
+            raise ValueError(f"gated_mlp: unknown activation {self.activation!r}")
+        # the up rows begin at a multiple of 8 rows, so that both halves of the product's rows stay aligned
+        self.up_at = -(-self.inter // 8) * 8
+        g, u = weights["gate"], weights["up"]
+        if g.dtype != u.dtype:
+            u = u.to(g.dtype)
+        stacked = torch.zeros((self.up_at + self.inter, self.hidden), dtype=g.dtype, device=g.device)
+        stacked[:self.inter] = g
+        stacked[self.up_at:] = u
+        self.gate_up = stacked
+        self.down = weights["down"]
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        return ProductRows.step_rows(rows, kind)
+
+    def tune(self, num_tokens: int) -> None:
+        n = int(num_tokens)
+        self.rt.tune_linear(self.rt.buffer("norm_out", (n, self.hidden)), self.gate_up)
+
+    def forward(self, x: torch.Tensor, out=None) -> torch.Tensor:
+        n, I = x.shape[0], self.inter
+        gu = self.rt.buffer("ffn_gate_up", (n, self.up_at + I))
+        ops.linear(x, self.gate_up, out=gu)
+        act = self.rt.buffer("ffn_act", (n, I))
+        ops.gated_act(gu[:, :I], gu[:, self.up_at:], self.activation, out=act)
+        if out is None:
+            out = self.rt.buffer("ffn_out", (n, self.hidden))
+        return ops.linear(act, self.down, out=out)
+
+
+@register_feed_forward("routed_experts")
+class RoutedExperts(FeedForward):
+    """A mixture of small feed-forwards down_e(gelu_erf(up_e(x))), no biases, of which every token uses ``top``.
+
+    Router: z = W_router x in float32, s = softmax(z) over all experts; the ``top`` experts with the largest
+    s + correction are chosen (the correction steers the choice only), their weights are s * ``scale``, not
+    renormalised; the result is the weighted sum of the chosen experts' outputs, in float32.
+
+    Everything runs on the device (``csrc/moe.hip``): the (token, choice) pairs are sorted by expert there, and the
+    two products walk tiles of rows of one expert each, so the launches of a step do not depend on what the
+    tokens choose.  The experts' matrices are stacked [E, ff, H] and [E, H, ff] at load.
+    params: hidden_size, experts, top, ff, scale."""
+
+    graph_safe = True
+    tape_safe = True
+    writes_into = True
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        H, E, ff = int(spec.params["hidden_size"]), int(spec.params["experts"]), int(spec.params["ff"])
+        w = {"router": WeightSpec((E, H)), "correction": WeightSpec((E,), init="zeros")}
+        for e in range(E):
+            w[f"up_{e}"] = WeightSpec((ff, H))
+            w[f"down_{e}"] = WeightSpec((H, ff))
+        return w
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden, self.experts, self.top, self.ff = int(p["hidden_size"]), int(p["experts"]), int(p["top"]), int(p["ff"])
+        self.scale = float(p.get("scale", 1.0))
+        if not (0 < self.top <= self.experts):
+            raise ValueError(f"routed_experts: top {self.top} of {self.experts} experts")
+        self.router = weights["router"]
+        self.correction = weights["correction"].float().contiguous()
+        self.up = torch.stack([weights[f"up_{e}"] for e in range(self.experts)]).contiguous()
+        self.down = torch.stack([weights[f"down_{e}"] for e in range(self.experts)]).contiguous()
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        return ProductRows.step_rows(rows, kind)
+
+    def forward(self, x: torch.Tensor, out=None) -> torch.Tensor:
+        n, E, top, rt = x.shape[0], self.experts, self.top, self.rt
+        pairs = n * top
+        z = ops.linear(x, self.router, out=rt.buffer("moe_logits", (n, E), torch.float32))
+        idx = rt.buffer("moe_choice", (n, top), torch.int32)
+        wt = rt.buffer("moe_weight", (n, top), torch.float32)
+        ops.moe_route(z, self.correction, top, self.scale, idx, wt)
+        rows = ops.moe_tile_rows(x.dtype, self.up.dtype, (self.hidden, self.ff), pairs, E)
+        tiles = ops.moe_max_tiles(pairs, E, rows)
+        plan = rt.buffer("moe_plan", (1 + 3 * tiles,), torch.int32)
+        order = rt.buffer("moe_order", (pairs,), torch.int32)
+        place_of = rt.buffer("moe_place", (pairs,), torch.int32)
+        ops.moe_group(idx, E, rows, plan, order, place_of)
+        act = rt.buffer("moe_act", (pairs, self.ff))
+        ops.moe_linear(x, self.up, plan, rows, tiles, out=act, source=order, source_div=top, activation="gelu_erf")
+        y = rt.buffer("moe_out_rows", (pairs, self.hidden), torch.float32)
+        ops.moe_linear(act, self.down, plan, rows, tiles, out=y)
+        if out is None:
+            out = rt.buffer("moe_out", (n, self.hidden), torch.float32)
+        return ops.moe_combine(y, wt, place_of, out)

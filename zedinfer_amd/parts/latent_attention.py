@@ -1,0 +1,101 @@
+"""Latent attention: keys and values made from one short latent per token."""
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from .. import ops
+from ..config.forward_config import PartSpec
+from ..weights.loader import WeightSpec
+from .base import (PAGE, KVCacheRequest, LayerMemory, Mixer, PageTensor, POSITION_ENCODINGS, Runtime, register_mixer)
+from .rows import ProductRows
+
+
+def latent_cache_request(kind: str, rank: int, rot: int, window: int = 0) -> KVCacheRequest:
+    """What latent attention keeps in a page: the normed latents [slot][rank] and the rotated key parts
+    [slot][rot] that all heads share."""
+    return KVCacheRequest(kind, int(window), (("latent", PageTensor((PAGE, int(rank)))),
+                                              ("key_part", PageTensor((PAGE, int(rot))))))
+
+
+@register_mixer("latent_attention")
+class LatentAttention(Mixer):
+    """Causal softmax attention, over all keys or a sliding window, whose keys and values are made from a latent.
+
+    Per token: (d_1 .. d_rank+rot) = W_dkv x; c = rms_norm(d_1..rank) * g is the latent, the last ``rot`` values,
+    turned by the position, are a key part kr shared by all heads.  Head h's query is (q_plain [dim], q_rot [rot],
+    turned), its key for token j (W_uk_h c_j, kr_j), its value W_uv_h c_j; score = (q . k) * scale; the window lets
+    position i see j with 0 <= i - j < window.  Only c and kr are cached.  The kernels never make keys or values:
+    q_plain is carried through W_uk_h once a token and head, the attended latents through W_uv_h afterwards
+    (``csrc/latent.hip``).  Scores, softmax and the sums over positions are float32; the cache holds the
+    activation type.
+
+    A layer built with ``shares_cache`` has no W_dkv: its run of the schedule names the cache of the layer whose
+    latents it reads (``ScheduleStep.writes_cache`` False), and it brings its own W_uk, W_uv, queries, window.
+
+    params: hidden_size, heads, dim, rot_dim, vdim, kv_rank, scale, window (0: all keys), eps, shares_cache,
+    position (a PartSpec of an encoding that hands over ``pair_table``: neighbouring pairs turn)."""
+
+    graph_safe = True
+    tape_safe = True
+    padding_safe = True      # padding has no place in the cache and no real token sees it
+    writes_into = True
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        p = spec.params
+        H, nh, dim, rot, vdim, rank = (int(p[k]) for k in ("hidden_size", "heads", "dim", "rot_dim", "vdim", "kv_rank"))
+        w = {"q": WeightSpec((nh * (dim + rot), H)), "uk": WeightSpec((nh * dim, rank)),
+             "uv": WeightSpec((nh * vdim, rank)), "o": WeightSpec((H, nh * vdim))}
+        if not p.get("shares_cache", False):
+            w["dkv"] = WeightSpec((rank + rot, H))
+            w["dkv_norm"] = WeightSpec((rank,), init="ones")
+        return w
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden, self.nh, self.dim, self.rot, self.vdim, self.rank = (
+            int(p[k]) for k in ("hidden_size", "heads", "dim", "rot_dim", "vdim", "kv_rank"))
+        self.scale = float(p["scale"])
+        self.window = int(p.get("window", 0) or 0)
+        self.eps = float(p.get("eps", 1e-6))
+        self.shares_cache = bool(p.get("shares_cache", False))
+        if self.rot % 2:
+            raise ValueError(f"latent_attention: rot_dim {self.rot} must be even")
+        pos_spec: PartSpec = p["position"]
+        self.position = POSITION_ENCODINGS.get(pos_spec.kind)(pos_spec, {}, rt)
+        if self.rot and (not hasattr(self.position, "pair_table") or self.position.rotary_dim != self.rot):
+            raise ValueError("latent_attention: the position encoding must turn neighbouring pairs of all rot_dim dims")
+        self.q, self.uk, self.uv, self.o = weights["q"], weights["uk"], weights["uv"], weights["o"]
+        if not self.shares_cache:
+            self.dkv = weights["dkv"]
+            self.dkv_norm = weights["dkv_norm"]
+
+    def cache_request(self) -> Optional[KVCacheRequest]:
+        return latent_cache_request("window" if self.window > 0 else "full", self.rank, self.rot, self.window)
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        return ProductRows.step_rows(rows, kind)
+
+    def forward(self, x: torch.Tensor, batch, memory: LayerMemory, out=None) -> torch.Tensor:
+        n, rt = x.shape[0], self.rt
+        view = batch.groups[memory.group]
+        table = self.position.pair_table(batch) if self.rot else None
+        c_cache, kr_cache = memory.tensors["latent"], memory.tensors["key_part"]
+        if memory.writes:
+            if self.shares_cache:
+                raise ValueError("latent_attention: a layer without W_dkv cannot write a cache")
+            dkv = ops.linear(x, self.dkv, out=rt.buffer("latent_dkv", (n, self.rank + self.rot), torch.float32))
+            ops.latent_store(dkv, self.dkv_norm, self.eps, table, view.slots, c_cache, kr_cache, self.rank, self.rot)
+        q = ops.linear(x, self.q, out=rt.buffer("latent_q", (n, self.nh * (self.dim + self.rot)), torch.float32))
+        qa = rt.buffer("latent_qa", (n, self.nh, self.rank + self.rot), torch.float32)
+        ops.latent_query(q, self.uk, table, self.nh, self.dim, self.rank, self.rot, out=qa)
+        o = rt.buffer("latent_attended", (n, self.nh, self.rank), torch.float32)
+        ops.latent_attention(qa, c_cache, kr_cache, batch.tok_seq, batch.positions, view.block_tables, self.scale,
+                             self.window, out=o)
+        heads = ops.latent_value(o, self.uv, self.vdim, out=rt.buffer("latent_heads", (n, self.nh * self.vdim)))
+        if out is None:
+            out = rt.buffer("latent_out", (n, self.hidden))
+        return ops.linear(heads, self.o, out=out)

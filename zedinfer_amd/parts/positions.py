@@ -3,6 +3,7 @@ from __future__ import annotations
 
 from typing import Dict
 
+import numpy as np
 import torch
 
 from .. import ops
@@ -43,6 +44,46 @@ class RopeNeox(PositionEncoding):
         table = ops.rope_table(positions, self.inv_freq)
         ops.rope_kv_store(q, None, None, table, None, None, None, nh, nkv, d)
         ops.rope_kv_store(k, None, None, table, None, None, None, nkv, nkv, d)
+
+
+@register_position_encoding("rope_pairs")
+class RopePairs(PositionEncoding):
+    """Rotary encoding over neighbouring pairs: dims (2i, 2i + 1) of the first R = ``rotary_dim`` dims of each head
+    turn by pos * theta^(-2i/R): (u, v) -> (u cos a - v sin a, v cos a + u sin a); the rest passes.
+    params: head_dim, theta, rotary_dim (default head_dim).
+
+    ``pair_table(batch)`` hands the step's (cos, sin) [n, R/2, 2] to mixers whose kernels turn pairs themselves;
+    ``step_table`` stays None, because mixers read that table as one of split halves."""
+
+    graph_safe = True
+    tape_safe = True
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        self.head_dim = int(spec.params["head_dim"])
+        self.rotary_dim = int(spec.params.get("rotary_dim", self.head_dim))
+        self.theta = float(spec.params["theta"])
+        if self.rotary_dim % 2 or not (0 < self.rotary_dim <= self.head_dim):
+            raise ValueError(f"rope_pairs: rotary_dim {self.rotary_dim} must be even and within head_dim {self.head_dim}")
+        if not self.theta > 0:
+            raise ValueError("rope_pairs: theta must be positive")
+        # the frequencies in double precision, rounded once
+        i = np.arange(self.rotary_dim // 2, dtype=np.float64)
+        self.inv_freq = torch.from_numpy(np.power(self.theta, -2.0 * i / self.rotary_dim).astype(np.float32)).to(rt.device)
+
+    def pair_table(self, batch):
+        key = ("rope_pairs", self.rotary_dim, self.theta)
+        table = batch.shared.get(key)
+        if table is None:
+            out = self.rt.buffer(f"rope_pairs_table_{self.rotary_dim}_{self.theta!r}",
+                                 (batch.num_tokens, self.rotary_dim // 2, 2), torch.float32)
+            table = batch.shared[key] = ops.rope_table(batch.positions, self.inv_freq, out=out)
+        return table
+
+    def encode(self, q, k, positions, nh: int, nkv: int, d: int) -> None:
+        table = ops.rope_table(positions, self.inv_freq)
+        ops.rope_pairs(q, table, nh, d)
+        ops.rope_pairs(k, table, nkv, d)
 
 
 @register_position_encoding("none")
