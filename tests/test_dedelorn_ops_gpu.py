@@ -358,3 +358,72 @@ def test_experts_products_over_the_sorted_pairs(dtype, n, experts, top, H, ff):
             e = int(idx[t, j])
             want[t] += float(wt[t, j]) * (plain.gelu_erf(x[t].double() @ up[e].double().t()) @ down[e].double().t())
     _close(out, want, 3e-5 if dtype == torch.float32 else 2e-2, "experts")
+
+
+@pytest.mark.parametrize("rank, rot", [(40, 8), (136, 24), (264, 16)])
+@pytest.mark.parametrize("window, page_size", [(0, 8), (13, 8), (64, 16), (150, 4)])
+@pytest.mark.parametrize("waves, chunk_keys", [(1, 0), (4, 0), (1, 128), (4, 128)])
+def test_latent_attention_on_the_matrix_cores(rank, rot, window, page_size, waves, chunk_keys):
+    """A prompt's portion of 37 tokens (tiles that end inside a token's heads, and a last tile with rows to spare)
+    beside a decoded token of another sequence, over shuffled pages of one pool; every cut of the keys and both
+    workgroup sizes against the plain sums; the keys at the window's edge planted as for the plain kernel."""
+    ops = _ops()
+    if chunk_keys and not window:
+        pytest.skip("keys are cut only under a window")
+    g = torch.Generator().manual_seed(rank + window)
+    H, scale, dtype = 5, 0.5, torch.bfloat16
+    T = [140, 77]
+    c = [(0.3 * torch.randn(t, rank, generator=g)).to(dtype) for t in T]
+    kr = [(0.3 * torch.randn(t, rot, generator=g)).to(dtype) for t in T]
+    past, lens = [103, 76], [37, 1]
+    n = sum(lens)
+    qa = torch.randn(n, H, rank + rot, generator=g)
+    W = window if window else 10 ** 6
+    for e, row in ((0, 36), (1, 37)):                               # the last token of either entry
+        p = past[e] + lens[e] - 1
+        direction = qa[row, 0, :rank] / qa[row, 0, :rank].norm()
+        if p - W + 1 >= 0:
+            c[e][p - W + 1] = (6.0 * direction).to(dtype)
+        if p - W >= 0:
+            c[e][p - W] = (12.0 * direction).to(dtype)
+    pages = 80
+    perm = torch.randperm(pages, generator=g)
+    cc = torch.full((pages, page_size, rank), 9e3, dtype=dtype)
+    kk = torch.full((pages, page_size, rot), 9e3, dtype=dtype)
+    width = -(-max(T) // page_size) + 3
+    bt = torch.full((2, width), -1, dtype=torch.int32)
+    at = 0
+    for e in range(2):
+        for j in range(T[e]):
+            if j % page_size == 0:
+                bt[e, j // page_size] = perm[at]
+                at += 1
+            cc[bt[e, j // page_size], j % page_size] = c[e][j]
+            kk[bt[e, j // page_size], j % page_size] = kr[e][j]
+    want = torch.cat([_plain_attend(qa[:37].to(dtype).float(), c[0].float(), kr[0].float(), list(range(103, 140)), window, scale),
+                      _plain_attend(qa[37:].to(dtype).float(), c[1].float(), kr[1].float(), [76], window, scale)])
+    chunks = 1
+    if chunk_keys:
+        chunks = -(-(window + -(-16 * waves // H) + 1) // chunk_keys)
+        if chunks == 1:
+            chunk_keys = 0
+    need = ops.latent_attention_cores_workspace(n, H, rank, chunks)
+    ws = torch.full((max(need, 1),), float("nan"), device=DEV)
+    out = torch.full((n, H, rank), float("nan"), device=DEV)
+    ops.latent_attention_cores(qa.to(DEV), cc.to(DEV), kk.to(DEV), _i32([0, 37]), _i32(lens), _i32(past), bt.to(DEV), scale,
+                               window, out=out, waves=waves, chunk_keys=chunk_keys, chunks=chunks, workspace=ws)
+    _close(out, want, 1.5e-2, f"rank {rank} window {window} waves {waves} chunks {chunks}")
+    # and against the plain kernel on the same cache
+    plain_out = torch.empty_like(out)
+    ops.latent_attention(qa.to(DEV), cc.to(DEV), kk.to(DEV), _i32([0] * 37 + [1]), _i32(list(range(103, 140)) + [76]),
+                         bt.to(DEV), scale, window, out=plain_out)
+    _close(out, plain_out, 1.5e-2, "against the plain kernel")
+
+
+def test_latent_attention_cores_plan_is_a_function_of_the_shape():
+    ops = _ops()
+    assert ops.latent_attention_cores_plan(2048, 1, 12, 1024, 256) == (4, 0, 1)          # a prompt fills the chip uncut
+    waves, keys, chunks = ops.latent_attention_cores_plan(8, 8, 12, 1024, 256)           # decoded tokens: cut
+    assert waves == 1 and keys == 128 and chunks * keys >= 1024 + 3
+    assert ops.latent_attention_cores_plan(8, 8, 12, 0, 256) == (1, 0, 1)                # no window, no cut
+    assert ops.latent_attention_cores_plan(8, 8, 12, 72, 256) == (1, 0, 1)               # a window of one chunk

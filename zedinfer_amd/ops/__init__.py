@@ -19,7 +19,8 @@ from .functional import (add, add_rms_norm, argmax, attention, attention_decode,
                          rope_kv_store, rope_kv_store_sums, rope_table, sample, swiglu, swiglu_t,
                          DECODE_LAYER_SPIN_LIMIT, FEW_ROWS, SUMS_MAX_ROWS)
 from .mixing import (delta_conv_state, delta_prepare, delta_rule, delta_state_floats, gated_act, gated_rms_norm,
-                     latent_attention, latent_query, latent_store, latent_value, moe_combine, moe_group, moe_linear,
+                     latent_attention, latent_attention_cores, latent_attention_cores_plan,
+                     latent_attention_cores_supported, latent_attention_cores_workspace, latent_query, latent_store, latent_value, moe_combine, moe_group, moe_linear,
                      moe_max_tiles, moe_route, moe_tile_rows, rope_pairs)
 from ._lib import KernelLibraryError, library_path, load
 
@@ -35,7 +36,8 @@ __all__ = [
     "linear_swiglu_supported", "linear_transposed", "linear_tune", "reduce_sums", "rms_norm", "rope",
     "rope_inv_freq", "rope_kv_store", "rope_kv_store_sums", "rope_table", "sample", "swiglu", "swiglu_t",
     "delta_conv_state", "delta_prepare", "delta_rule", "delta_state_floats", "gated_act", "gated_rms_norm",
-    "latent_attention", "latent_query", "latent_store", "latent_value", "moe_combine", "moe_group", "moe_linear",
+    "latent_attention", "latent_attention_cores", "latent_attention_cores_plan", "latent_attention_cores_supported",
+    "latent_attention_cores_workspace", "latent_query", "latent_store", "latent_value", "moe_combine", "moe_group", "moe_linear",
     "moe_max_tiles", "moe_route", "moe_tile_rows", "rope_pairs",
     "KernelLibraryError", "library_path", "load", "FEW_ROWS", "SUMS_MAX_ROWS",
 ]

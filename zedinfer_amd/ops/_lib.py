@@ -70,6 +70,9 @@ _PROTOTYPES = {
     "zi_latent_store": [P, I, L, I, P, I, F, P, P, P, P, L, I, I, P],
     "zi_latent_query": [P, P, I, L, P, I, P, I, I, I, I, I, P],
     "zi_latent_attention": [P, P, P, P, I, I, P, P, P, P, I, I, I, I, I, I, I, F, P],
+    "zi_latent_attention_cores": [P, P, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, I, I, I, P],
+    "zi_latent_attention_cores_supported": [I, I, I],
+    "zi_latent_attention_cores_tiles": [I, I, I, I],
     "zi_latent_value": [P, I, L, P, P, I, I, I, I, I, P],
     "zi_delta_prepare": [P, P, P, P, L, I, P, P, P, I, P, L, L, P, P, P, I, I, I, I, I, P],
     "zi_delta_conv_state": [P, L, L, P, L, P, P, P, I, I, I, P],

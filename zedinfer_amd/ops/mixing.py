@@ -131,6 +131,70 @@ def latent_attention(qa: torch.Tensor, c_cache: torch.Tensor, kr_cache: torch.Te
     return out
 
 
+LATENT_CHUNK_KEYS = 128      # keys of a chunk when a tile's keys are cut over workgroups
+
+
+def latent_attention_cores_supported(cache_dtype: torch.dtype, rank: int, rot: int) -> bool:
+    """Whether the matrix-core kernel takes caches of this type and these sizes."""
+    if cache_dtype != torch.bfloat16:
+        return False
+    return bool(_lib.load().zi_latent_attention_cores_supported(1, int(rank), int(rot)))
+
+
+def latent_attention_cores_plan(n: int, entries: int, heads: int, window: int, units: int):
+    """(wavefronts a workgroup, keys a chunk, chunks) for a step of n tokens in ``entries`` entries: 64 rows a
+    workgroup when that many tiles fill the chip, else 16; a tile's keys are cut into chunks when the tiles alone
+    are fewer than the chip's compute units (decoded tokens, short portions) and a window bounds them.  A function of the step's shape."""
+    lib = _lib.load()
+    waves = 4 if lib.zi_latent_attention_cores_tiles(int(n), int(entries), int(heads), 4) >= units else 1
+    tiles = lib.zi_latent_attention_cores_tiles(int(n), int(entries), int(heads), waves)
+    if window > 0 and tiles < units:
+        span = int(window) + -(-16 * waves // int(heads)) + 1
+        chunks = -(-span // LATENT_CHUNK_KEYS)
+        if chunks > 1:
+            return waves, LATENT_CHUNK_KEYS, chunks
+    return waves, 0, 1
+
+
+def latent_attention_cores_workspace(n: int, heads: int, rank: int, chunks: int) -> int:
+    """Floats of workspace for the chunks' partial results (0 without a cut)."""
+    return int(chunks) * int(n) * int(heads) * (int(rank) + 2) if chunks > 1 else 0
+
+
+def latent_attention_cores(qa: torch.Tensor, c_cache: torch.Tensor, kr_cache: torch.Tensor, entry_start: torch.Tensor,
+                           entry_len: torch.Tensor, entry_past: torch.Tensor, block_tables: torch.Tensor, scale: float,
+                           window: int, out: torch.Tensor, waves: int = 1, chunk_keys: int = 0, chunks: int = 1,
+                           workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """``latent_attention`` on the matrix cores, for all tokens of a step (bfloat16 caches): entry e brings the
+    tokens entry_start[e] ... of positions entry_past[e] ...; queries are rounded to bfloat16 for the products,
+    scores, softmax and sums are float32."""
+    _gpu("latent_attention_cores", qa, c_cache, kr_cache, entry_start, entry_len, entry_past, block_tables, out, workspace)
+    if qa.dim() != 3:
+        raise ValueError("latent_attention_cores: qa must be [n, heads, rank + rot]")
+    n, heads, qw = qa.shape
+    rank = int(c_cache.shape[2]) if c_cache.dim() == 3 else -1
+    rot = qw - rank
+    pages, ps = _latent_caches(c_cache, kr_cache, rank, rot, "latent_attention_cores")
+    if not latent_attention_cores_supported(c_cache.dtype, rank, rot):
+        raise ValueError(f"latent_attention_cores: a {c_cache.dtype} cache with rank {rank} and rot {rot} is not taken")
+    _f32(qa, "latent_attention_cores qa")
+    _f32(out, "latent_attention_cores out", (n, heads, rank))
+    E = entry_start.numel()
+    for t in (entry_start, entry_len, entry_past):
+        _i32(t, "latent_attention_cores entries", E)
+    if block_tables.dim() != 2 or block_tables.shape[0] < E:
+        raise ValueError("latent_attention_cores: block tables must be [entries, pages]")
+    _i32(block_tables, "latent_attention_cores block_tables")
+    need = latent_attention_cores_workspace(n, heads, rank, chunks)
+    if need and (workspace is None or workspace.dtype != torch.float32 or workspace.numel() < need):
+        raise ValueError(f"latent_attention_cores: {need} floats of workspace are needed")
+    _lib.call("zi_latent_attention_cores", _p(out), _p(workspace), int(workspace.numel()) if workspace is not None else 0,
+              _p(qa), _p(c_cache), _p(kr_cache), _p(entry_start), _p(entry_len), _p(entry_past), _p(block_tables), E, n,
+              int(block_tables.shape[1]), pages, heads, rank, rot, ps, int(window), float(scale), int(waves),
+              int(chunk_keys), int(chunks), _stream())
+    return out
+
+
 def latent_value(o: torch.Tensor, w_uv: torch.Tensor, vdim: int, out: torch.Tensor) -> torch.Tensor:
     """out [n, heads * vdim] = every head's attended latent o [n, heads, rank] through its block of ``w_uv``
     [heads * vdim, rank]."""

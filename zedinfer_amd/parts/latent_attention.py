@@ -69,6 +69,10 @@ class LatentAttention(Mixer):
         if self.rot and (not hasattr(self.position, "pair_table") or self.position.rotary_dim != self.rot):
             raise ValueError("latent_attention: the position encoding must turn neighbouring pairs of all rot_dim dims")
         self.q, self.uk, self.uv, self.o = weights["q"], weights["uk"], weights["uv"], weights["o"]
+        # a bfloat16 cache of sizes the matrix-core kernel takes goes there; everything else to the plain kernel
+        self.cores = (rt.device.type == "cuda" and rt.dtype == torch.bfloat16
+                      and ops.latent_attention_cores_supported(rt.dtype, self.rank, self.rot))
+        self.units = ops.compute_units() if rt.device.type == "cuda" else 256
         if not self.shares_cache:
             self.dkv = weights["dkv"]
             self.dkv_norm = weights["dkv_norm"]
@@ -93,8 +97,16 @@ class LatentAttention(Mixer):
         qa = rt.buffer("latent_qa", (n, self.nh, self.rank + self.rot), torch.float32)
         ops.latent_query(q, self.uk, table, self.nh, self.dim, self.rank, self.rot, out=qa)
         o = rt.buffer("latent_attended", (n, self.nh, self.rank), torch.float32)
-        ops.latent_attention(qa, c_cache, kr_cache, batch.tok_seq, batch.positions, view.block_tables, self.scale,
-                             self.window, out=o)
+        if self.cores:
+            waves, chunk_keys, chunks = ops.latent_attention_cores_plan(n, batch.num_entries, self.nh, self.window, self.units)
+            need = ops.latent_attention_cores_workspace(n, self.nh, self.rank, chunks)
+            ws = rt.buffer("latent_chunks", (need,), torch.float32) if need else None
+            ops.latent_attention_cores(qa, c_cache, kr_cache, batch.entry_start, batch.entry_len, batch.entry_past,
+                                       view.block_tables, self.scale, self.window, out=o, waves=waves,
+                                       chunk_keys=chunk_keys, chunks=chunks, workspace=ws)
+        else:
+            ops.latent_attention(qa, c_cache, kr_cache, batch.tok_seq, batch.positions, view.block_tables, self.scale,
+                                 self.window, out=o)
         heads = ops.latent_value(o, self.uv, self.vdim, out=rt.buffer("latent_heads", (n, self.nh * self.vdim)))
         if out is None:
             out = rt.buffer("latent_out", (n, self.hidden))
