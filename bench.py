@@ -17,6 +17,7 @@ uniform random in [100, vocab-100] as in the reference's own benchmark
 import argparse
 import gc
 import json
+import math
 import os
 import random
 import sys
@@ -375,6 +376,90 @@ def resident_layer_probe(args, shape):
     return 0
 
 
+# ---- another design beside the benchmark's architecture (--design) -------------------------------------------------
+# Layer sizes that resemble a real model's, for the Dedelorn design: three gated-delta-rule layers, then one of
+# latent attention under a window of 1,024 keys (every second of those reads the latents of the one before it);
+# dense feed-forwards alternate with routed experts.
+DESIGN_SIZES = {
+    "1.5B": dict(width=1536, heads=12, ff=8960, experts=32, top=4, expert_ff=1536),
+    "7B": dict(width=3584, heads=28, ff=18944, experts=32, top=4, expert_ff=2560),
+}
+
+
+def dedelorn_shape(size, layers, vocab):
+    z = DESIGN_SIZES[size]
+    out, last_latent = [], None
+    for i in range(layers):
+        if i % 4 == 3:
+            mixer = dict(heads=z["heads"], dim=128, rot_dim=64, vdim=128, kv_rank=512, scale=192 ** -0.5,
+                         mask=dict(size=1024), rot=dict(base=10000.0, dims=64))
+            if last_latent is not None:
+                mixer["kv_from"] = last_latent
+                last_latent = None
+            else:
+                last_latent = i
+            kind = "latent_attention"
+        else:
+            mixer = dict(heads=z["heads"], kv_heads=z["heads"] // 2, dim=128, vdim=128, conv=4)
+            kind = "delta"
+        mlp = dict(kind="dense", ff=z["ff"]) if i % 2 == 0 else \
+            dict(kind="moe", expert=dict(ff=z["expert_ff"]), router=dict(experts=z["experts"], top=z["top"], scale=1.0))
+        out.append(dict(type=kind, mixer=mixer, mlp=mlp))
+    return dict(architecture="Dedelorn", width=z["width"], vocab=vocab, norm=dict(eps=1e-6), layers=out)
+
+
+def design_comparison(args):
+    """Prefill and decode of a model of the design at a real model's layer sizes, and of the benchmark's own
+    architecture (Qwen2 dense) at the same width, layers, heads and dense feed-forward, one after the other."""
+    import torch
+    from zedinfer_amd.config import DedelornConfig, Qwen2Config, SchedulerConfig
+    from zedinfer_amd.engine import Engine
+    layers = args.layers if args.layers != FULL_LAYERS else 8
+    vocab, prompt = 32000, args.prompt_len
+    result = {"metric": f"{args.design} beside Qwen2 dense at equal layer sizes", "dtype": args.dtype, "layers_run": layers,
+              "data": "synthetic: seeded random weights, seeded uniform-random token ids", "sizes": {}}
+    for size in (args.design_sizes.split(",") if args.design_sizes else ["1.5B"]):
+        z = DESIGN_SIZES[size]
+        models = {
+            "dedelorn": (DedelornConfig.from_dict(dedelorn_shape(size, layers, vocab)), "Dedelorn"),
+            "qwen2": (Qwen2Config.from_dict(dict(SHAPE, hidden_size=z["width"], intermediate_size=z["ff"], vocab_size=vocab,
+                                                 num_hidden_layers=layers, num_attention_heads=z["heads"],
+                                                 num_key_value_heads=max(2, z["heads"] // 7), tie_word_embeddings=False)),
+                      "Qwen2ForCausalLM"),
+        }
+        rec = {}
+        for name, (cfg, arch) in models.items():
+            cache = {}
+
+            def factory(batch):
+                def make():
+                    tokens = prompt + args.warmup + args.steps + 2 * batch + 64
+                    sched = SchedulerConfig(num_kv_blocks=batch * (-(-tokens // 16)) + 16, kv_block_size=16,
+                                            max_batch_requests=max(batch, 1), max_batch_tokens=prompt + batch,
+                                            max_prefill_tokens=prompt, max_seq_len=max(CONTEXT, 2 * prompt))
+                    if "e" not in cache:
+                        cache["e"] = Engine.from_config(cfg, arch, args.dtype, seed=0, sched=sched)
+                        return cache["e"]
+                    return cache["e"].with_cache(sched)
+                return make
+            one = {}
+            for tokens in (512, args.prefill_len):
+                ms = measure_prefill(factory(1), vocab, tokens=tokens)
+                one[f"prefill_{tokens}"] = {"ms": round(ms, 3), "tok_s": round(tokens / ms * 1000.0, 1)}
+            for batch, steps in ((8, args.steps), (64, min(args.steps, 32))):
+                tps, ms_step, _ = measure_decode(factory(batch), batch, steps, min(args.warmup, 8), vocab, prompt)
+                one[f"decode_b{batch}"] = {"tok_s": round(tps, 1), "ms_per_step": round(ms_step, 4)}
+            from zedinfer_amd.models import expected_weights
+            one["parameters"] = int(sum(math.prod(ws.shape) for ws in expected_weights(cache["e"].fc).values()))
+            rec[name] = one
+            cache.clear()
+            gc.collect()
+            torch.cuda.empty_cache()
+        result["sizes"][size] = rec
+    print(json.dumps(result))
+    return 0
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -395,6 +480,11 @@ def main():
                     help="run only the 2,048-token prefill (for profiling) and print its figures")
     ap.add_argument("--resident-layer", action="store_true",
                     help="instead: time the one-launch decoder layer (ops.decode_layer) alone, --layers launches a step")
+    ap.add_argument("--design", default="", choices=["", "dedelorn"],
+                    help="instead: prefill and decode of a model of this design at a real model's layer sizes, beside "
+                         "Qwen2 dense of equal sizes (8 layers unless --layers says otherwise)")
+    ap.add_argument("--design-sizes", default="", help="with --design: layer sizes, of " + ", ".join(sorted(DESIGN_SIZES)) +
+                    " (commas between them; default 1.5B)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -411,6 +501,8 @@ def main():
     shape["num_hidden_layers"] = args.layers
     if args.resident_layer:
         return resident_layer_probe(args, shape)
+    if args.design:
+        return design_comparison(args)
     cfg = Qwen2Config.from_dict(shape)
     el = 2 if args.dtype == "bf16" else 4
     weights_cache = {}

@@ -17,44 +17,60 @@ __device__ __forceinline__ float delta_silu(float z) { return z / (1.f + expf(-z
 __device__ __forceinline__ float delta_softplus(float z) { return z > 30.f ? z : log1pf(expf(z)); }
 
 // proj [n][ld]: columns [q (kvh*dim) | k (kvh*dim) | v (heads*vdim) | gate (heads*vdim) | b (heads) | a (heads)].
-// One workgroup per token.
-template <typename TW>
-__global__ void __launch_bounds__(256)
+// One workgroup per (token, unit): a unit is one head of q or k (its dim channels, and their unit length), or 256
+// channels of v; the first unit of a token also makes its beta and g.
+#define DELTA_UNIT 256
+
+__device__ __forceinline__ float delta_conv(const float* __restrict__ proj, int64_t ld, const float* __restrict__ conv_w,
+                                            const float* __restrict__ tail, int t, int local, int c, int C, int taps) {
+    float y = 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int li = local - (taps - 1) + j;
+        const float x = li >= 0 ? proj[(int64_t)(t - local + li) * ld + c] : tail[(int64_t)(li + taps - 1) * C + c];
+        y += conv_w[(int64_t)c * taps + j] * x;
+    }
+    return delta_silu(y);
+}
+
+__global__ void __launch_bounds__(DELTA_UNIT)
 delta_prepare_kernel(float* __restrict__ qk, float* __restrict__ v, float* __restrict__ beta_g,
-                     const float* __restrict__ proj, int64_t ld, const TW* __restrict__ conv_w,
-                     const TW* __restrict__ a_log, const TW* __restrict__ dt_bias, const float* __restrict__ state,
+                     const float* __restrict__ proj, int64_t ld, const float* __restrict__ conv_w,
+                     const float* __restrict__ a_log, const float* __restrict__ dt_bias, const float* __restrict__ state,
                      int64_t state_stride, int64_t conv_off, const int32_t* __restrict__ tok_seq,
                      const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_slot, int heads,
                      int kvh, int dim, int vdim, int taps) {
-    extern __shared__ float act[];      // [channels]
-    const int t = blockIdx.x, e = tok_seq[t];
+    __shared__ float red[16];
+    const int t = blockIdx.x, unit = blockIdx.y, e = tok_seq[t];
     const int local = t - entry_start[e];
     const int qkc = 2 * kvh * dim, C = qkc + heads * vdim;
     const float* tail = state + (int64_t)entry_slot[e] * state_stride + conv_off;      // [taps - 1][C]
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
-        float y = 0.f;
-        for (int j = 0; j < taps; ++j) {
-            const int li = local - (taps - 1) + j;
-            const float x = li >= 0 ? proj[(int64_t)(t - local + li) * ld + c] : tail[(int64_t)(li + taps - 1) * C + c];
-            y += zi_load(conv_w + (int64_t)c * taps + j) * x;
+    if (unit < 2 * kvh) {
+        // dim may exceed the workgroup: a thread takes channels threadIdx.x, threadIdx.x + 256, ...
+        float x[2] = {0.f, 0.f}, ss = 0.f;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int d = threadIdx.x + i * DELTA_UNIT;
+            if (d < dim) x[i] = delta_conv(proj, ld, conv_w, tail, t, local, unit * dim + d, C, taps);
+            ss += x[i] * x[i];
         }
-        act[c] = delta_silu(y);
+        ss = zi_block_sum(ss, red);
+        const float r = (1.f / sqrtf(ss + 1e-6f)) * (unit < kvh ? 1.f / sqrtf((float)dim) : 1.f);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int d = threadIdx.x + i * DELTA_UNIT;
+            if (d < dim) qk[(int64_t)t * qkc + unit * dim + d] = x[i] * r;
+        }
+    } else {
+        const int c = (unit - 2 * kvh) * DELTA_UNIT + threadIdx.x;
+        if (c < heads * vdim) v[(int64_t)t * heads * vdim + c] = delta_conv(proj, ld, conv_w, tail, t, local, qkc + c, C, taps);
     }
-    __syncthreads();
-    const int lane = threadIdx.x % ZI_WAVE, wave = threadIdx.x / ZI_WAVE, waves = blockDim.x / ZI_WAVE;
-    for (int hd = wave; hd < 2 * kvh; hd += waves) {       // the heads of q, then those of k
-        float ss = 0.f;
-        for (int d = lane; d < dim; d += ZI_WAVE) ss += act[hd * dim + d] * act[hd * dim + d];
-        ss = zi_wave_sum(ss);
-        const float r = (1.f / sqrtf(ss + 1e-6f)) * (hd < kvh ? 1.f / sqrtf((float)dim) : 1.f);
-        for (int d = lane; d < dim; d += ZI_WAVE) qk[(int64_t)t * qkc + hd * dim + d] = act[hd * dim + d] * r;
-    }
-    for (int c = threadIdx.x; c < heads * vdim; c += blockDim.x) v[(int64_t)t * heads * vdim + c] = act[qkc + c];
-    const float* row = proj + (int64_t)t * ld + C + heads * vdim;      // b, then a
-    for (int h = threadIdx.x; h < heads; h += blockDim.x) {
-        beta_g[(int64_t)t * 2 * heads + h] = 1.f / (1.f + expf(-row[h]));
-        const float step = delta_softplus(row[heads + h] + zi_load(dt_bias + h));
-        beta_g[(int64_t)t * 2 * heads + heads + h] = expf(-expf(zi_load(a_log + h)) * step);
+    if (unit == 0) {
+        const float* row = proj + (int64_t)t * ld + C + heads * vdim;      // b, then a
+        for (int h = threadIdx.x; h < heads; h += blockDim.x) {
+            beta_g[(int64_t)t * 2 * heads + h] = 1.f / (1.f + expf(-row[h]));
+            const float step = delta_softplus(row[heads + h] + dt_bias[h]);
+            beta_g[(int64_t)t * 2 * heads + heads + h] = expf(-expf(a_log[h]) * step);
+        }
     }
 }
 
@@ -65,16 +81,17 @@ extern "C" int zi_delta_prepare(float* qk, float* v, float* beta_g, const float*
                                 hipStream_t stream) {
     ZI_REQUIRE(n >= 0 && heads > 0 && kvh > 0 && heads % kvh == 0 && dim > 0 && vdim > 0 && taps >= 1,
                "delta_prepare: bad sizes");
+    ZI_REQUIRE(w_dt == ZI_F32, "delta_prepare: the convolution's taps, A_log and dt_bias are float32");
+    ZI_REQUIRE(dim <= 2 * DELTA_UNIT, "delta_prepare: dim %d is more than %d", dim, 2 * DELTA_UNIT);
     const int64_t C = 2LL * kvh * dim + (int64_t)heads * vdim;
     ZI_REQUIRE(ld >= C + (int64_t)heads * vdim + 2 * heads, "delta_prepare: row stride too small");
-    ZI_REQUIRE(C * sizeof(float) <= 64 * 1024, "delta_prepare: %lld channels are more than a workgroup holds", (long long)C);
     ZI_REQUIRE(state_stride >= conv_off + (int64_t)(taps - 1) * C, "delta_prepare: the state row is too short");
+    const int units = 2 * kvh + (heads * vdim + DELTA_UNIT - 1) / DELTA_UNIT;
+    ZI_REQUIRE(units <= 65535, "delta_prepare: too many channels");
     if (n == 0) return 0;
-    ZI_DISPATCH_DTYPE(w_dt, TW, {
-        delta_prepare_kernel<TW><<<n, 256, C * sizeof(float), stream>>>(
-            qk, v, beta_g, proj, ld, (const TW*)conv_w, (const TW*)a_log, (const TW*)dt_bias, state, state_stride, conv_off,
-            tok_seq, entry_start, entry_slot, heads, kvh, dim, vdim, taps);
-    });
+    delta_prepare_kernel<<<dim3(n, units), DELTA_UNIT, 0, stream>>>(
+        qk, v, beta_g, proj, ld, (const float*)conv_w, (const float*)a_log, (const float*)dt_bias, state, state_stride,
+        conv_off, tok_seq, entry_start, entry_slot, heads, kvh, dim, vdim, taps);
     return zi_check_launch("delta_prepare");
 }
 
@@ -122,10 +139,12 @@ extern "C" int zi_delta_conv_state(float* state, int64_t state_stride, int64_t c
 
 // The recurrence.  One wavefront per (entry, head, 16 columns of S): lane (col, part) holds rows part, part + 4,
 // part + 8, ... of column col, so a dot product over dim is a quarter of it in every lane and two lane exchanges.
-// The order of the additions is fixed by dim alone.  k and q of TOKS tokens at a time are brought into LDS.
+// The order of the additions is fixed by dim alone.  q, k, v, beta and g of TOKS tokens at a time lie in LDS; the
+// next TOKS tokens' are requested before the present ones are worked on and put into the other LDS buffer
+// afterwards, so no token waits for memory.
 #define DELTA_COLS 16
 #define DELTA_PARTS 4
-#define DELTA_TOKS 16
+#define DELTA_TOKS 8
 
 template <int R>      // rows a lane holds: dim <= 4 R
 __global__ void __launch_bounds__(ZI_WAVE)
@@ -133,10 +152,12 @@ delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qk, const f
                   const float* __restrict__ beta_g, float* __restrict__ state, int64_t state_stride,
                   const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
                   const int32_t* __restrict__ entry_slot, int heads, int kvh, int dim, int vdim) {
-    __shared__ float ks[DELTA_TOKS][4 * R], qs[DELTA_TOKS][4 * R];
-    __shared__ float bg[DELTA_TOKS][2];
+    constexpr int D = 4 * R, PRE = DELTA_TOKS * D * 2 / ZI_WAVE, PRE_V = DELTA_TOKS * DELTA_COLS / ZI_WAVE;
+    __shared__ float qks[2][2][DELTA_TOKS][D];      // [buffer][q, k][token][d]
+    __shared__ float vs[2][DELTA_TOKS][DELTA_COLS];
+    __shared__ float bg[2][DELTA_TOKS][2];
     const int e = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
-    const int col = blockIdx.x * DELTA_COLS + lane % DELTA_COLS, part = lane / DELTA_COLS;
+    const int col0 = blockIdx.x * DELTA_COLS, col = col0 + lane % DELTA_COLS, part = lane / DELTA_COLS;
     const bool live = col < vdim;
     const int kh = h / (heads / kvh), qkc = 2 * kvh * dim;
     const int start = entry_start[e], len = entry_len[e];
@@ -147,27 +168,49 @@ delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qk, const f
         const int d = part + DELTA_PARTS * i;
         s[i] = (live && d < dim) ? S[(int64_t)d * vdim + col] : 0.f;
     }
-    for (int t0 = 0; t0 < len; t0 += DELTA_TOKS) {
-        const int cnt = len - t0 < DELTA_TOKS ? len - t0 : DELTA_TOKS;
-        __syncthreads();
-        for (int i = lane; i < cnt * dim; i += ZI_WAVE) {
-            const int tt = i / dim, d = i % dim;
-            const float* row = qk + (int64_t)(start + t0 + tt) * qkc;
-            qs[tt][d] = row[kh * dim + d];
-            ks[tt][d] = row[(kvh + kh) * dim + d];
+    float pre[PRE], pre_v[PRE_V], pre_bg = 0.f;
+    // request the tokens t0 .. t0 + TOKS - 1 of the entry (those past its end: nothing)
+    auto request = [&](int t0) {
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int idx = lane + ZI_WAVE * i, which = idx / (DELTA_TOKS * D), tt = (idx / D) % DELTA_TOKS, d = idx % D;
+            pre[i] = (t0 + tt < len && d < dim) ? qk[(int64_t)(start + t0 + tt) * qkc + (which * kvh + kh) * dim + d] : 0.f;
         }
-        if (lane < 2 * cnt) bg[lane / 2][lane % 2] = beta_g[(int64_t)(start + t0 + lane / 2) * 2 * heads + (lane % 2) * heads + h];
-        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < PRE_V; ++i) {
+            const int idx = lane + ZI_WAVE * i, tt = idx / DELTA_COLS, c = col0 + idx % DELTA_COLS;
+            pre_v[i] = (t0 + tt < len && c < vdim) ? v[((int64_t)(start + t0 + tt) * heads + h) * vdim + c] : 0.f;
+        }
+        if (lane < 2 * DELTA_TOKS)
+            pre_bg = t0 + lane / 2 < len ? beta_g[(int64_t)(start + t0 + lane / 2) * 2 * heads + (lane % 2) * heads + h] : 0.f;
+    };
+    auto put = [&](int buf) {
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int idx = lane + ZI_WAVE * i;
+            (&qks[buf][0][0][0])[idx] = pre[i];
+        }
+#pragma unroll
+        for (int i = 0; i < PRE_V; ++i) (&vs[buf][0][0])[lane + ZI_WAVE * i] = pre_v[i];
+        if (lane < 2 * DELTA_TOKS) (&bg[buf][0][0])[lane] = pre_bg;
+    };
+    request(0);
+    put(0);
+    __syncthreads();
+    int buf = 0;
+    for (int t0 = 0; t0 < len; t0 += DELTA_TOKS, buf ^= 1) {
+        const int cnt = len - t0 < DELTA_TOKS ? len - t0 : DELTA_TOKS;
+        if (t0 + DELTA_TOKS < len) request(t0 + DELTA_TOKS);
         for (int tt = 0; tt < cnt; ++tt) {
-            const int t = start + t0 + tt;
-            const float beta = bg[tt][0], g = bg[tt][1];
-            const float vv = live ? v[((int64_t)t * heads + h) * vdim + col] : 0.f;
+            const float beta = bg[buf][tt][0], g = bg[buf][tt][1];
+            const float vv = vs[buf][tt][lane % DELTA_COLS];
+            const float* kk = qks[buf][1][tt];
+            const float* qq = qks[buf][0][tt];
             float dot = 0.f;
 #pragma unroll
             for (int i = 0; i < R; ++i) {
-                const int d = part + DELTA_PARTS * i;
                 s[i] *= g;
-                if (d < dim) dot += s[i] * ks[tt][d];
+                dot += s[i] * kk[part + DELTA_PARTS * i];      // rows past dim hold zeros, and meet zeros
             }
             dot += __shfl_xor(dot, 16, ZI_WAVE);
             dot += __shfl_xor(dot, 32, ZI_WAVE);
@@ -175,16 +218,15 @@ delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qk, const f
             float o = 0.f;
 #pragma unroll
             for (int i = 0; i < R; ++i) {
-                const int d = part + DELTA_PARTS * i;
-                if (d < dim) {
-                    s[i] += ks[tt][d] * u;
-                    o += s[i] * qs[tt][d];
-                }
+                s[i] += kk[part + DELTA_PARTS * i] * u;
+                o += s[i] * qq[part + DELTA_PARTS * i];
             }
             o += __shfl_xor(o, 16, ZI_WAVE);
             o += __shfl_xor(o, 32, ZI_WAVE);
-            if (live && part == 0) out[((int64_t)t * heads + h) * vdim + col] = o;
+            if (live && part == 0) out[((int64_t)(start + t0 + tt) * heads + h) * vdim + col] = o;
         }
+        if (t0 + DELTA_TOKS < len) put(buf ^ 1);
+        __syncthreads();
     }
 #pragma unroll
     for (int i = 0; i < R; ++i) {

@@ -34,6 +34,7 @@ union la_pack {
 #define LA_BK 32      // keys a block
 #define LA_PAD 8      // elements of padding of an LDS row
 #define LA_EMPTY -1e30f
+#define LA_BATCH 6     // requests a thread has in flight while it stages a block
 
 template <int WAVES, int NT, int KS>      // rank <= 16 NT, rank + rot <= 32 KS
 __global__ void __launch_bounds__(WAVES* ZI_WAVE)
@@ -103,27 +104,39 @@ latent_attention_cores_kernel(float* __restrict__ out, float* __restrict__ parti
     constexpr int G = KD / 8;      // pieces of eight of a staged key
     for (int kb = k_lo; kb <= k_hi; kb += LA_BK) {
         __syncthreads();
-        for (int i = threadIdx.x; i < LA_BK * G; i += WAVES * ZI_WAVE) {
-            const int key = i / G, d = (i % G) * 8, kp = kb + key;
-            la_pack val;
-            val.u = (la_u32x4_t){0u, 0u, 0u, 0u};
-            if (kp <= k_hi && d < qw) {
-                const int pi = kp / page_size;
-                const int page = pi < max_pages ? bt[pi] : -1;
-                if ((unsigned)page < (unsigned)num_pages) {
-                    const int64_t slot = (int64_t)page * page_size + kp % page_size;
-                    val.u = d < rank ? *reinterpret_cast<const la_u32x4_t*>(c_cache + slot * rank + d)
-                                     : *reinterpret_cast<const la_u32x4_t*>(kr_cache + slot * rot + (d - rank));
-                }
-            }
-            *reinterpret_cast<la_u32x4_t*>(&krow[key * KP + d]) = val.u;
-            if (d < RD) {
-                const unsigned keep = d < rank ? 0xffffffffu : 0u;      // the key parts are no values
+        // requests in batches of LA_BATCH a thread, all of a batch before the first is put into LDS
+        for (int i0 = threadIdx.x; i0 < LA_BK * G; i0 += WAVES * ZI_WAVE * LA_BATCH) {
+            la_pack val[LA_BATCH];
 #pragma unroll
-                for (int x = 0; x < 4; ++x) {
-                    const unsigned w = val.w[x] & keep;
-                    ct[(d + 2 * x) * CP + key] = (uint16_t)(w & 0xffffu);
-                    ct[(d + 2 * x + 1) * CP + key] = (uint16_t)(w >> 16);
+            for (int u = 0; u < LA_BATCH; ++u) {
+                const int i = i0 + u * WAVES * ZI_WAVE;
+                const int key = (i / G) % LA_BK, d = (i % G) * 8, kp = kb + key;
+                // addresses are clamped, not guarded (a load under a branch would make every load before it
+                // wait), and what was read for a place that does not exist is masked
+                const bool want = i < LA_BK * G && kp <= k_hi && d < qw;
+                const int kc = kp <= k_hi ? kp : k_hi, dc = d < qw ? d : 0;
+                const int pi = kc / page_size;
+                const int page = bt[pi < max_pages ? pi : max_pages - 1];
+                const bool held = (unsigned)page < (unsigned)num_pages;
+                const int64_t slot = (int64_t)(held ? page : 0) * page_size + kc % page_size;
+                const zi_bf16* src = dc < rank ? c_cache + slot * rank + dc : kr_cache + slot * rot + (dc - rank);
+                const unsigned mask = 0u - (unsigned)(want && held);
+                val[u].u = *reinterpret_cast<const la_u32x4_t*>(src) & mask;
+            }
+#pragma unroll
+            for (int u = 0; u < LA_BATCH; ++u) {
+                const int i = i0 + u * WAVES * ZI_WAVE;
+                if (i >= LA_BK * G) break;
+                const int key = i / G, d = (i % G) * 8;
+                *reinterpret_cast<la_u32x4_t*>(&krow[key * KP + d]) = val[u].u;
+                if (d < RD) {
+                    const unsigned keep = d < rank ? 0xffffffffu : 0u;      // the key parts are no values
+#pragma unroll
+                    for (int x = 0; x < 4; ++x) {
+                        const unsigned w = val[u].w[x] & keep;
+                        ct[(d + 2 * x) * CP + key] = (uint16_t)(w & 0xffffu);
+                        ct[(d + 2 * x + 1) * CP + key] = (uint16_t)(w >> 16);
+                    }
                 }
             }
         }
@@ -287,4 +300,90 @@ extern "C" int zi_latent_attention_cores(float* out, float* partial, int64_t par
     if (rc != 0 || chunks == 1) return rc;
     latent_attention_merge_kernel<<<total_rows, 256, 0, stream>>>(out, partial, chunks, total_rows, rank);
     return zi_check_launch("latent_attention_merge");
+}
+
+// ---- a product per head on the matrix cores ---------------------------------------------------------------------
+// out[t][h][i] = sum_k w[h][i][k] x[t][h][k]: w bfloat16 [heads][N][K] (k runs fastest), x float32 with row stride
+// ldx and head stride xs (rounded to bfloat16 as it is loaded), out float32 or bfloat16 with row stride ldo and head
+// stride os.  One wavefront per (16 tokens, head, 16 outputs); operands straight from memory.  It carries the
+// queries through W_uk (w = W_uk of the head, transposed at load) and the attended latents through W_uv.
+template <typename TO>
+__global__ void __launch_bounds__(ZI_WAVE)
+headwise_linear_cores_kernel(TO* __restrict__ out, int64_t ldo, int os, const float* __restrict__ x, int64_t ldx, int xs,
+                             const zi_bf16* __restrict__ w, int n, int N, int K) {
+    const int t0 = blockIdx.x * 16, h = blockIdx.y, n0 = blockIdx.z * 16;
+    const int lane = threadIdx.x, r = lane % 16, j = lane / 16;
+    const zi_bf16* wrow = w + ((int64_t)h * N + (n0 + r < N ? n0 + r : N - 1)) * K;
+    const float* xrow = x + (int64_t)(t0 + r < n ? t0 + r : n - 1) * ldx + (int64_t)h * xs;
+    la_f32x4_t acc = (la_f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const int k = k0 + 8 * j;
+        const bool in = k < K;      // K is a multiple of 8
+        const int kc = in ? k : 0;
+        const unsigned mask = 0u - (unsigned)in;
+        la_pack a, b;
+        a.u = *reinterpret_cast<const la_u32x4_t*>(wrow + kc) & mask;
+        const float4 lo = *reinterpret_cast<const float4*>(xrow + kc), hi = *reinterpret_cast<const float4*>(xrow + kc + 4);
+        b.w[0] = zi_pack_bf16x2(lo.x, lo.y) & mask;
+        b.w[1] = zi_pack_bf16x2(lo.z, lo.w) & mask;
+        b.w[2] = zi_pack_bf16x2(hi.x, hi.y) & mask;
+        b.w[3] = zi_pack_bf16x2(hi.z, hi.w) & mask;
+        acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b.b, acc, 0, 0, 0);
+    }
+    if (t0 + r >= n) return;
+    TO* orow = out + (int64_t)(t0 + r) * ldo + (int64_t)h * os + n0 + 4 * j;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (n0 + 4 * j + i < N) zi_store(orow + i, acc[i]);
+}
+
+extern "C" int zi_headwise_linear_supported(int w_dt, int K, int64_t ldx, int xs) {
+    return w_dt == ZI_BF16 && K > 0 && K % 8 == 0 && ldx % 4 == 0 && xs % 4 == 0;
+}
+
+extern "C" int zi_headwise_linear(void* out, int out_dt, int64_t ldo, int os, const float* x, int64_t ldx, int xs,
+                                  const void* w, int n, int heads, int N, int K, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && heads > 0 && heads <= 65535 && N > 0 && (N + 15) / 16 <= 65535, "headwise_linear: bad sizes");
+    ZI_REQUIRE(zi_headwise_linear_supported(ZI_BF16, K, ldx, xs) && ((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0,
+               "headwise_linear: K %d, row stride %lld, head stride %d or an address is not aligned", K, (long long)ldx, xs);
+    ZI_REQUIRE(xs >= K && os >= N && ldx >= (int64_t)(heads - 1) * xs + K && ldo >= (int64_t)(heads - 1) * os + N,
+               "headwise_linear: strides too small");
+    if (n == 0) return 0;
+    const dim3 grid((n + 15) / 16, heads, (N + 15) / 16);
+    ZI_DISPATCH_DTYPE(out_dt, TO, {
+        headwise_linear_cores_kernel<TO><<<grid, ZI_WAVE, 0, stream>>>((TO*)out, ldo, os, x, ldx, xs, (const zi_bf16*)w, n, N, K);
+    });
+    return zi_check_launch("headwise_linear");
+}
+
+// qa[t][h][rank + ...] = the rotated part of every head's query, turned in neighbouring pairs.
+template <typename T>
+__global__ void latent_query_rot_kernel(float* __restrict__ qa, const T* __restrict__ q, int64_t ldq,
+                                        const float* __restrict__ table, int n, int heads, int dim, int rank, int rot) {
+    const int half = rot / 2;
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)n * heads * half) return;
+    const int p = (int)(i % half), h = (int)((i / half) % heads);
+    const int64_t t = i / ((int64_t)half * heads);
+    const T* qr = q + t * ldq + (int64_t)h * (dim + rot) + dim + 2 * p;
+    const float u = zi_load(qr), v = zi_load(qr + 1);
+    const float c = table[(t * half + p) * 2], s = table[(t * half + p) * 2 + 1];
+    float* o = qa + (t * heads + h) * (rank + rot) + rank + 2 * p;
+    o[0] = u * c - v * s;
+    o[1] = v * c + u * s;
+}
+
+extern "C" int zi_latent_query_rot(float* qa, const void* q, int dt, int64_t ldq, const float* table, int n, int heads,
+                                   int dim, int rank, int rot, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && heads > 0 && dim > 0 && rank > 0 && rot >= 0 && rot % 2 == 0 && ldq >= (int64_t)heads * (dim + rot),
+               "latent_query_rot: bad sizes");
+    const int64_t total = (int64_t)n * heads * (rot / 2);
+    if (total == 0) return 0;
+    ZI_REQUIRE(table, "latent_query_rot: no table of angles");
+    ZI_DISPATCH_DTYPE(dt, T, {
+        latent_query_rot_kernel<T><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(qa, (const T*)q, ldq, table, n, heads,
+                                                                                         dim, rank, rot);
+    });
+    return zi_check_launch("latent_query_rot");
 }

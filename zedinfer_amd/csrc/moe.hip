@@ -233,6 +233,7 @@ moe_linear_mfma_kernel(TO* __restrict__ out, int64_t ldo, const zi_bf16* __restr
     moe_f32x4_t acc[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) acc[t] = (moe_f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
     for (int k0 = 0; k0 < K; k0 += 32) {
         const int k = k0 + 8 * j;
         const bool in = k < K;      // K is a multiple of 8: a piece of eight lies inside or outside

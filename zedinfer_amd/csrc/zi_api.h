@@ -109,6 +109,12 @@ int zi_latent_attention_cores(float* out, float* partial, int64_t partial_floats
     const void* kr_cache, const int32_t* entry_start, const int32_t* entry_len, const int32_t* entry_past, const int32_t*
     block_tables, int entries, int n, int max_pages, int num_pages, int heads, int rank, int rot, int page_size, int
     window, float scale, int waves, int chunk_keys, int chunks, hipStream_t stream);
+// latent_cores.hip
+int zi_headwise_linear(void* out, int out_dt, int64_t ldo, int os, const float* x, int64_t ldx, int xs, const void* w, int
+    n, int heads, int N, int K, hipStream_t stream);
+// latent_cores.hip
+int zi_latent_query_rot(float* qa, const void* q, int dt, int64_t ldq, const float* table, int n, int heads, int dim, int
+    rank, int rot, hipStream_t stream);
 // latent.hip
 int zi_latent_value(void* out, int out_dt, int64_t ldo, const float* o, const void* w_uv, int w_dt, int n, int heads,
     int vdim, int rank, hipStream_t stream);
@@ -179,6 +185,8 @@ int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int ro
     X(zi_latent_query) \
     X(zi_latent_attention) \
     X(zi_latent_attention_cores) \
+    X(zi_headwise_linear) \
+    X(zi_latent_query_rot) \
     X(zi_latent_value) \
     X(zi_delta_prepare) \
     X(zi_delta_conv_state) \

@@ -73,6 +73,9 @@ _PROTOTYPES = {
     "zi_latent_attention_cores": [P, P, L, P, P, P, P, P, P, P, I, I, I, I, I, I, I, I, I, F, I, I, I, P],
     "zi_latent_attention_cores_supported": [I, I, I],
     "zi_latent_attention_cores_tiles": [I, I, I, I],
+    "zi_headwise_linear": [P, I, L, I, P, L, I, P, I, I, I, I, P],
+    "zi_headwise_linear_supported": [I, I, L, I],
+    "zi_latent_query_rot": [P, P, I, L, P, I, I, I, I, I, P],
     "zi_latent_value": [P, I, L, P, P, I, I, I, I, I, P],
     "zi_delta_prepare": [P, P, P, P, L, I, P, P, P, I, P, L, L, P, P, P, I, I, I, I, I, P],
     "zi_delta_conv_state": [P, L, L, P, L, P, P, P, I, I, I, P],

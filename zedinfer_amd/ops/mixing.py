@@ -84,7 +84,7 @@ def latent_store(dkv: torch.Tensor, norm_w: torch.Tensor, eps: float, table: Opt
 
 
 def latent_query(q: torch.Tensor, w_uk: torch.Tensor, table: Optional[torch.Tensor], heads: int, dim: int, rank: int,
-                 rot: int, out: torch.Tensor) -> torch.Tensor:
+                 rot: int, out: torch.Tensor, w_uk_t: Optional[torch.Tensor] = None) -> torch.Tensor:
     """out [n, heads, rank + rot] float32: every head's unrotated query part carried through its block of
     ``w_uk`` [heads * dim, rank] (so that it meets latents instead of keys), then its rotated part, turned."""
     _gpu("latent_query", q, w_uk, table, out)
@@ -97,6 +97,17 @@ def latent_query(q: torch.Tensor, w_uk: torch.Tensor, table: Optional[torch.Tens
     _f32(out, "latent_query out", (n, heads, rank + rot))
     if rot:
         _f32(table, "latent_query table", (n, rot // 2, 2))
+    if w_uk_t is not None and q.dtype == torch.float32 and q.data_ptr() % 16 == 0 \
+            and _lib.load().zi_headwise_linear_supported(_code(w_uk_t, "latent_query w_uk_t"), dim, ldq, dim + rot):
+        # on the matrix cores: the head's block of W_uk, transposed at load, times the unrotated query parts
+        if tuple(w_uk_t.shape) != (heads, rank, dim) or not w_uk_t.is_contiguous():
+            raise ValueError(f"latent_query: w_uk_t must be a contiguous [{heads}, {rank}, {dim}] tensor")
+        _lib.call("zi_headwise_linear", _p(out), 0, heads * (rank + rot), rank + rot, _p(q), ldq, dim + rot, _p(w_uk_t), n,
+                  heads, rank, dim, _stream())
+        if rot:
+            _lib.call("zi_latent_query_rot", _p(out), _p(q), _code(q, "latent_query q"), ldq, _p(table), n, heads, dim, rank,
+                      rot, _stream())
+        return out
     _lib.call("zi_latent_query", _p(out), _p(q), _code(q, "latent_query q"), ldq, _p(w_uk), _code(w_uk, "latent_query w_uk"),
               _p(table), n, heads, dim, rank, rot, _stream())
     return out
@@ -206,6 +217,11 @@ def latent_value(o: torch.Tensor, w_uv: torch.Tensor, vdim: int, out: torch.Tens
     ldo, width = _rows(out, "latent_value out")
     if tuple(out.shape) != (n, heads * vdim):
         raise ValueError(f"latent_value: out must be [{n}, {heads * vdim}]")
+    if w_uv.dtype == torch.bfloat16 and _lib.load().zi_headwise_linear_supported(1, rank, heads * rank, rank) \
+            and w_uv.data_ptr() % 16 == 0:
+        _lib.call("zi_headwise_linear", _p(out), _code(out, "latent_value out"), ldo, vdim, _p(o), heads * rank, rank,
+                  _p(w_uv), n, heads, vdim, rank, _stream())
+        return out
     _lib.call("zi_latent_value", _p(out), _code(out, "latent_value out"), ldo, _p(o), _p(w_uv), _code(w_uv, "latent_value w_uv"),
               n, heads, vdim, rank, _stream())
     return out

@@ -73,6 +73,10 @@ class LatentAttention(Mixer):
         self.cores = (rt.device.type == "cuda" and rt.dtype == torch.bfloat16
                       and ops.latent_attention_cores_supported(rt.dtype, self.rank, self.rot))
         self.units = ops.compute_units() if rt.device.type == "cuda" else 256
+        # the heads' blocks of W_uk with the contraction running fastest, for the matrix cores
+        self.uk_t = None
+        if self.uk.dtype == torch.bfloat16 and self.dim % 8 == 0:
+            self.uk_t = self.uk.view(self.nh, self.dim, self.rank).transpose(1, 2).contiguous()
         if not self.shares_cache:
             self.dkv = weights["dkv"]
             self.dkv_norm = weights["dkv_norm"]
@@ -95,7 +99,7 @@ class LatentAttention(Mixer):
             ops.latent_store(dkv, self.dkv_norm, self.eps, table, view.slots, c_cache, kr_cache, self.rank, self.rot)
         q = ops.linear(x, self.q, out=rt.buffer("latent_q", (n, self.nh * (self.dim + self.rot)), torch.float32))
         qa = rt.buffer("latent_qa", (n, self.nh, self.rank + self.rot), torch.float32)
-        ops.latent_query(q, self.uk, table, self.nh, self.dim, self.rank, self.rot, out=qa)
+        ops.latent_query(q, self.uk, table, self.nh, self.dim, self.rank, self.rot, out=qa, w_uk_t=self.uk_t)
         o = rt.buffer("latent_attended", (n, self.nh, self.rank), torch.float32)
         if self.cores:
             waves, chunk_keys, chunks = ops.latent_attention_cores_plan(n, batch.num_entries, self.nh, self.window, self.units)
