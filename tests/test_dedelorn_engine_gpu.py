@@ -169,3 +169,35 @@ def test_the_replay_tool_runs_a_model_of_the_design(tmp_path):
         _check(steps, out, ref, requests, dtype, "tool")
         said = open(str(tmp_path / f"err_{dtype}.txt")).read()
         assert "4 live requests" in said
+
+
+def test_command_lines_take_a_model_of_the_design(tmp_path):
+    """random_model writes a folder from the design's config.json, ping generates from it what the plain implementation
+    generates, batch_bench runs its scheduler over it with random weights."""
+    import json
+    import subprocess
+    import sys
+    ROOT = traces.ROOT
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    run = lambda *a: subprocess.run([sys.executable, *a], capture_output=True, text=True, env=env, timeout=300,  # noqa: E731
+                                    cwd=str(tmp_path))
+    (tmp_path / "cfg").mkdir()
+    with open(tmp_path / "cfg" / "config.json", "w") as f:
+        json.dump(models.ALL, f)
+    folder = str(tmp_path / "made")
+    r = run(os.path.join(ROOT, "bin", "random_model"), str(tmp_path / "cfg"), folder, "--seed", "5", "--dtype", "float32",
+            "--std", "0.1", "--noisy-norms")
+    assert r.returncode == 0 and "Dedelorn" in r.stdout, r.stderr
+    with open(os.path.join(folder, "config.json")) as f:
+        assert json.load(f) == models.ALL
+    cfg, w = plain.load_folder(folder, torch.float64)
+    assert set(w) == set(models.tensor_shapes(models.ALL))
+    prompt = traces.random_tokens(cfg["vocab"], 27, seed=3)
+    r = run(os.path.join(ROOT, "bin", "ping"), folder, "--dtype", "fp32", "--prompt-ids", ",".join(map(str, prompt)),
+            "--max-new-tokens", "6", "--ignore-eos", "--num-kv-blocks", "32", "--kv-block-size", "8", "--no-log-to-console")
+    assert r.returncode == 0, r.stderr
+    want = plain.greedy_generate(cfg, w, prompt, 6)
+    assert "output_ids: " + ",".join(map(str, want)) in r.stdout, r.stdout
+    r = run(os.path.join(ROOT, "bin", "batch_bench"), str(tmp_path / "cfg"), "-b", "3", "-p", "20", "-d", "6", "--num-kv-blocks",
+            "64", "--kv-block-size", "8", "--random-weights", "--seed", "4", "--no-log-to-console")
+    assert r.returncode == 0 and "18 tokens generated" in r.stdout, r.stderr + r.stdout

@@ -137,27 +137,49 @@ extern "C" int zi_delta_conv_state(float* state, int64_t state_stride, int64_t c
     return zi_check_launch("delta_conv_state");
 }
 
-// The recurrence.  One wavefront per (entry, head, 16 columns of S): lane (col, part) holds rows part, part + 4,
-// part + 8, ... of column col, so a dot product over dim is a quarter of it in every lane and two lane exchanges.
-// The order of the additions is fixed by dim alone.  q, k, v, beta and g of TOKS tokens at a time lie in LDS; the
-// next TOKS tokens' are requested before the present ones are worked on and put into the other LDS buffer
-// afterwards, so no token waits for memory.
-#define DELTA_COLS 16
-#define DELTA_PARTS 4
+// The recurrence.  One wavefront per (entry, head, 8 columns of S): lane (col, part) = 8 col + part holds the R rows
+// part R ... part R + R - 1 of column col, so a dot product over dim is an eighth of it in every lane and three
+// exchanges among 8 neighbouring lanes (data-parallel-primitive moves, no trip through LDS).  (Sixteen parts and 4
+// columns a wavefront were measured too: a prompt of 2,048 tokens 1.07 against 1.22 ms a layer, but decoded tokens
+// 23 against 14 us, the state then being read in pieces of 16 bytes.)
+// With S the state before the token, the token's read-out needs no second pass over the updated state:
+//     a = S^T k,  b = S^T q   (two dot products over the same registers, reduced together)
+//     u = beta (v - g a);     o = g b + (k . q) u;     S <- g S + k u^T
+// which is the rule's S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q with the products regrouped.  k . q
+// does not depend on the state: it is made when the tokens are put into LDS.  The order of all additions is fixed
+// by dim alone.  q, k, v, beta and g of TOKS tokens at a time lie in LDS; the next TOKS tokens' are requested
+// before the present ones are worked on and put into the other LDS buffer afterwards, so no token waits for memory.
+#define DELTA_COLS 8
+#define DELTA_PARTS 8
 #define DELTA_TOKS 8
 
-template <int R>      // rows a lane holds: dim <= 4 R
+// x of the lane that `ctrl` names within this lane's row of 16 (quad permutations, mirrors)
+template <int CTRL>
+__device__ __forceinline__ float delta_dpp(float x) {
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, true));
+}
+// the sum over the 8 lanes of a half row, in every one of them: neighbours, pairs of neighbours, the other quad of
+// the half (lane 7 - i)
+__device__ __forceinline__ float delta_row_sum(float x) {
+    x += delta_dpp<0xB1>(x);       // quad_perm [1, 0, 3, 2]
+    x += delta_dpp<0x4E>(x);       // quad_perm [2, 3, 0, 1]
+    x += delta_dpp<0x141>(x);      // row_half_mirror
+    return x;
+}
+
+template <int R>      // rows a lane holds: dim <= 8 R; R is a multiple of 4
 __global__ void __launch_bounds__(ZI_WAVE)
 delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qk, const float* __restrict__ v,
                   const float* __restrict__ beta_g, float* __restrict__ state, int64_t state_stride,
                   const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
                   const int32_t* __restrict__ entry_slot, int heads, int kvh, int dim, int vdim) {
-    constexpr int D = 4 * R, PRE = DELTA_TOKS * D * 2 / ZI_WAVE, PRE_V = DELTA_TOKS * DELTA_COLS / ZI_WAVE;
-    __shared__ float qks[2][2][DELTA_TOKS][D];      // [buffer][q, k][token][d]
+    constexpr int D = DELTA_PARTS * R, PRE = DELTA_TOKS * D * 2 / ZI_WAVE;
+    __shared__ __attribute__((aligned(16))) float qks[2][2][DELTA_TOKS][D];      // [buffer][q, k][token][d]
     __shared__ float vs[2][DELTA_TOKS][DELTA_COLS];
     __shared__ float bg[2][DELTA_TOKS][2];
+    __shared__ float kq[2][DELTA_TOKS];
     const int e = blockIdx.z, h = blockIdx.y, lane = threadIdx.x;
-    const int col0 = blockIdx.x * DELTA_COLS, col = col0 + lane % DELTA_COLS, part = lane / DELTA_COLS;
+    const int col0 = blockIdx.x * DELTA_COLS, col = col0 + lane / DELTA_PARTS, part = lane % DELTA_PARTS;
     const bool live = col < vdim;
     const int kh = h / (heads / kvh), qkc = 2 * kvh * dim;
     const int start = entry_start[e], len = entry_len[e];
@@ -165,34 +187,38 @@ delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qk, const f
     float s[R];
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-        const int d = part + DELTA_PARTS * i;
+        const int d = part * R + i;
         s[i] = (live && d < dim) ? S[(int64_t)d * vdim + col] : 0.f;
     }
-    float pre[PRE], pre_v[PRE_V], pre_bg = 0.f;
-    // request the tokens t0 .. t0 + TOKS - 1 of the entry (those past its end: nothing)
+    float pre[PRE], pre_v = 0.f, pre_bg = 0.f;
+    // request the tokens t0 .. t0 + TOKS - 1 of the entry (those past its end, and rows past dim: zeros)
     auto request = [&](int t0) {
 #pragma unroll
         for (int i = 0; i < PRE; ++i) {
             const int idx = lane + ZI_WAVE * i, which = idx / (DELTA_TOKS * D), tt = (idx / D) % DELTA_TOKS, d = idx % D;
             pre[i] = (t0 + tt < len && d < dim) ? qk[(int64_t)(start + t0 + tt) * qkc + (which * kvh + kh) * dim + d] : 0.f;
         }
-#pragma unroll
-        for (int i = 0; i < PRE_V; ++i) {
-            const int idx = lane + ZI_WAVE * i, tt = idx / DELTA_COLS, c = col0 + idx % DELTA_COLS;
-            pre_v[i] = (t0 + tt < len && c < vdim) ? v[((int64_t)(start + t0 + tt) * heads + h) * vdim + c] : 0.f;
+        if (lane < DELTA_TOKS * DELTA_COLS) {
+            const int tt = lane / DELTA_COLS, c = col0 + lane % DELTA_COLS;
+            pre_v = (t0 + tt < len && c < vdim) ? v[((int64_t)(start + t0 + tt) * heads + h) * vdim + c] : 0.f;
         }
         if (lane < 2 * DELTA_TOKS)
             pre_bg = t0 + lane / 2 < len ? beta_g[(int64_t)(start + t0 + lane / 2) * 2 * heads + (lane % 2) * heads + h] : 0.f;
     };
     auto put = [&](int buf) {
 #pragma unroll
-        for (int i = 0; i < PRE; ++i) {
-            const int idx = lane + ZI_WAVE * i;
-            (&qks[buf][0][0][0])[idx] = pre[i];
-        }
-#pragma unroll
-        for (int i = 0; i < PRE_V; ++i) (&vs[buf][0][0])[lane + ZI_WAVE * i] = pre_v[i];
+        for (int i = 0; i < PRE; ++i) (&qks[buf][0][0][0])[lane + ZI_WAVE * i] = pre[i];
+        if (lane < DELTA_TOKS * DELTA_COLS) (&vs[buf][0][0])[lane] = pre_v;
         if (lane < 2 * DELTA_TOKS) (&bg[buf][0][0])[lane] = pre_bg;
+        __syncthreads();
+        // k . q of the TOKS tokens: eight lanes a token
+        const int tt = lane / 8, sub = lane % 8;
+        float acc = 0.f;
+        for (int d = sub; d < D; d += 8) acc += qks[buf][0][tt][d] * qks[buf][1][tt][d];
+        acc += __shfl_xor(acc, 1, ZI_WAVE);
+        acc += __shfl_xor(acc, 2, ZI_WAVE);
+        acc += __shfl_xor(acc, 4, ZI_WAVE);
+        if (sub == 0) kq[buf][tt] = acc;
     };
     request(0);
     put(0);
@@ -202,35 +228,42 @@ delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qk, const f
         const int cnt = len - t0 < DELTA_TOKS ? len - t0 : DELTA_TOKS;
         if (t0 + DELTA_TOKS < len) request(t0 + DELTA_TOKS);
         for (int tt = 0; tt < cnt; ++tt) {
-            const float beta = bg[buf][tt][0], g = bg[buf][tt][1];
-            const float vv = vs[buf][tt][lane % DELTA_COLS];
-            const float* kk = qks[buf][1][tt];
-            const float* qq = qks[buf][0][tt];
-            float dot = 0.f;
+            const float beta = bg[buf][tt][0], g = bg[buf][tt][1], kqt = kq[buf][tt];
+            const float vv = vs[buf][tt][lane / DELTA_PARTS];
+            const float4* kk = reinterpret_cast<const float4*>(&qks[buf][1][tt][part * R]);
+            const float4* qq = reinterpret_cast<const float4*>(&qks[buf][0][tt][part * R]);
+            float4 kr[R / 4];
+            float a0 = 0.f, a1 = 0.f, b0 = 0.f, b1 = 0.f;
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                s[i] *= g;
-                dot += s[i] * kk[part + DELTA_PARTS * i];      // rows past dim hold zeros, and meet zeros
+            for (int i = 0; i < R / 4; ++i) {
+                kr[i] = kk[i];
+                const float4 q4 = qq[i];
+                a0 += s[4 * i] * kr[i].x;
+                a1 += s[4 * i + 1] * kr[i].y;
+                a0 += s[4 * i + 2] * kr[i].z;
+                a1 += s[4 * i + 3] * kr[i].w;
+                b0 += s[4 * i] * q4.x;
+                b1 += s[4 * i + 1] * q4.y;
+                b0 += s[4 * i + 2] * q4.z;
+                b1 += s[4 * i + 3] * q4.w;
             }
-            dot += __shfl_xor(dot, 16, ZI_WAVE);
-            dot += __shfl_xor(dot, 32, ZI_WAVE);
-            const float u = beta * (vv - dot);
-            float o = 0.f;
+            const float a = delta_row_sum(a0 + a1), b = delta_row_sum(b0 + b1);
+            const float u = beta * (vv - g * a);
+            if (live && part == 0) out[((int64_t)(start + t0 + tt) * heads + h) * vdim + col] = g * b + kqt * u;
 #pragma unroll
-            for (int i = 0; i < R; ++i) {
-                s[i] += kk[part + DELTA_PARTS * i] * u;
-                o += s[i] * qq[part + DELTA_PARTS * i];
+            for (int i = 0; i < R / 4; ++i) {
+                s[4 * i] = g * s[4 * i] + kr[i].x * u;
+                s[4 * i + 1] = g * s[4 * i + 1] + kr[i].y * u;
+                s[4 * i + 2] = g * s[4 * i + 2] + kr[i].z * u;
+                s[4 * i + 3] = g * s[4 * i + 3] + kr[i].w * u;
             }
-            o += __shfl_xor(o, 16, ZI_WAVE);
-            o += __shfl_xor(o, 32, ZI_WAVE);
-            if (live && part == 0) out[((int64_t)(start + t0 + tt) * heads + h) * vdim + col] = o;
         }
         if (t0 + DELTA_TOKS < len) put(buf ^ 1);
         __syncthreads();
     }
 #pragma unroll
     for (int i = 0; i < R; ++i) {
-        const int d = part + DELTA_PARTS * i;
+        const int d = part * R + i;
         if (live && d < dim) S[(int64_t)d * vdim + col] = s[i];
     }
 }
@@ -248,10 +281,10 @@ extern "C" int zi_delta_rule(float* out, const float* qk, const float* v, const 
 #define ZI_DELTA_RULE(R)                                                                                         \
     delta_rule_kernel<R><<<grid, ZI_WAVE, 0, stream>>>(out, qk, v, beta_g, state, state_stride, entry_start,      \
                                                        entry_len, entry_slot, heads, kvh, dim, vdim)
-    if (dim <= 32) ZI_DELTA_RULE(8);
-    else if (dim <= 64) ZI_DELTA_RULE(16);
-    else if (dim <= 128) ZI_DELTA_RULE(32);
-    else ZI_DELTA_RULE(64);
+    if (dim <= 32) ZI_DELTA_RULE(4);
+    else if (dim <= 64) ZI_DELTA_RULE(8);
+    else if (dim <= 128) ZI_DELTA_RULE(16);
+    else ZI_DELTA_RULE(32);
 #undef ZI_DELTA_RULE
     return zi_check_launch("delta_rule");
 }

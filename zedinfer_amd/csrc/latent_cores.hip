@@ -36,7 +36,9 @@ union la_pack {
 #define LA_EMPTY -1e30f
 #define LA_BATCH 6     // requests a thread has in flight while it stages a block
 
-template <int WAVES, int NT, int KS>      // rank <= 16 NT, rank + rot <= 32 KS
+// SPLIT: all WAVES wavefronts share one tile of 16 rows (decoded tokens): they stage together, each makes the
+// scores again (cheap) and every WAVES-th tile of 16 latent dims of the second product.
+template <int WAVES, int NT, int KS, bool SPLIT>      // rank <= 16 NT, rank + rot <= 32 KS
 __global__ void __launch_bounds__(WAVES* ZI_WAVE)
 latent_attention_cores_kernel(float* __restrict__ out, float* __restrict__ partial, const float* __restrict__ qa,
                               const zi_bf16* __restrict__ c_cache, const zi_bf16* __restrict__ kr_cache,
@@ -44,7 +46,7 @@ latent_attention_cores_kernel(float* __restrict__ out, float* __restrict__ parti
                               const int32_t* __restrict__ entry_past, const int32_t* __restrict__ block_tables,
                               int entries, int max_pages, int num_pages, int heads, int rank, int rot, int page_size,
                               int window, float scale, int chunk_keys, int total_rows) {
-    constexpr int ROWS = WAVES * 16, KD = KS * 32, KP = KD + LA_PAD, RD = NT * 16, CP = LA_BK + LA_PAD;
+    constexpr int ROWS = SPLIT ? 16 : WAVES * 16, OT = SPLIT ? (NT + WAVES - 1) / WAVES : NT, KD = KS * 32, KP = KD + LA_PAD, RD = NT * 16, CP = LA_BK + LA_PAD;
     __shared__ __attribute__((aligned(16))) uint16_t krow[LA_BK * KP];
     __shared__ __attribute__((aligned(16))) uint16_t ct[RD * CP];
     int tile = blockIdx.x, e = 0;
@@ -71,7 +73,7 @@ latent_attention_cores_kernel(float* __restrict__ out, float* __restrict__ parti
     }
 
     // this lane's row
-    const int row = row0 + wave * 16 + r;
+    const int row = row0 + (SPLIT ? 0 : wave * 16) + r;
     const bool row_ok = row < erows;
     const int rc = row_ok ? row : last_row;
     const int tok = start + rc / heads, head = rc % heads, pos = past + rc / heads;
@@ -97,9 +99,9 @@ latent_attention_cores_kernel(float* __restrict__ out, float* __restrict__ parti
     }
 
     float m = LA_EMPTY, l = 0.f;
-    la_f32x4_t o[NT];
+    la_f32x4_t o[OT];      // tile tq of this wavefront is the latent dims 16 t ..., t = tq (SPLIT: tq WAVES + wave)
 #pragma unroll
-    for (int t = 0; t < NT; ++t) o[t] = (la_f32x4_t){0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < OT; ++t) o[t] = (la_f32x4_t){0.f, 0.f, 0.f, 0.f};
 
     constexpr int G = KD / 8;      // pieces of eight of a staged key
     for (int kb = k_lo; kb <= k_hi; kb += LA_BK) {
@@ -187,13 +189,14 @@ latent_attention_cores_kernel(float* __restrict__ out, float* __restrict__ parti
         pb.w[2] = zi_pack_bf16x2(p[1][0], p[1][1]);
         pb.w[3] = zi_pack_bf16x2(p[1][2], p[1][3]);
 #pragma unroll
-        for (int t = 0; t < NT; ++t) {
+        for (int tq = 0; tq < OT; ++tq) {
+            const int t = SPLIT ? tq * WAVES + wave : tq;
             if (t * 16 < rank) {
-                o[t] *= corr;
+                o[tq] *= corr;
                 la_pack a;
                 a.h[0] = *reinterpret_cast<const la_u32x2_t*>(&ct[(t * 16 + r) * CP + 4 * j]);
                 a.h[1] = *reinterpret_cast<const la_u32x2_t*>(&ct[(t * 16 + r) * CP + 16 + 4 * j]);
-                o[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb.b, o[t], 0, 0, 0);
+                o[tq] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, pb.b, o[tq], 0, 0, 0);
             }
         }
     }
@@ -203,24 +206,24 @@ latent_attention_cores_kernel(float* __restrict__ out, float* __restrict__ parti
         const float inv = 1.f / l;
         float* orow = out + grow * rank;
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
+        for (int tq = 0; tq < OT; ++tq)
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
-                const int d = 16 * t + 4 * j + x;
-                if (d < rank) orow[d] = o[t][x] * inv;
+                const int d = 16 * (SPLIT ? tq * WAVES + wave : tq) + 4 * j + x;
+                if (d < rank) orow[d] = o[tq][x] * inv;
             }
     } else {
         float* prow = partial + ((int64_t)blockIdx.y * total_rows + grow) * (rank + 2);
-        if (j == 0) {
+        if (j == 0 && (!SPLIT || wave == 0)) {
             prow[0] = m;
             prow[1] = l;
         }
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
+        for (int tq = 0; tq < OT; ++tq)
 #pragma unroll
             for (int x = 0; x < 4; ++x) {
-                const int d = 16 * t + 4 * j + x;
-                if (d < rank) prow[2 + d] = o[t][x];
+                const int d = 16 * (SPLIT ? tq * WAVES + wave : tq) + 4 * j + x;
+                if (d < rank) prow[2 + d] = o[tq][x];
             }
     }
 }
@@ -283,7 +286,7 @@ extern "C" int zi_latent_attention_cores(float* out, float* partial, int64_t par
     const int total_rows = n * heads;
     const dim3 grid(zi_latent_attention_cores_tiles(n, entries, heads, waves), chunks);
 #define ZI_LA_LAUNCH(W, NT, KS)                                                                                       \
-    latent_attention_cores_kernel<W, NT, KS><<<grid, W * ZI_WAVE, 0, stream>>>(                                        \
+    latent_attention_cores_kernel<4, NT, KS, W == 1><<<grid, 4 * ZI_WAVE, 0, stream>>>(                                \
         out, partial, qa, (const zi_bf16*)c_cache, (const zi_bf16*)kr_cache, entry_start, entry_len, entry_past,       \
         block_tables, entries, max_pages, num_pages, heads, rank, rot, page_size, window, scale, chunk_keys, total_rows)
 #define ZI_LA_SIZES(W)                                                       \
