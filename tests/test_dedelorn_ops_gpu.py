@@ -427,6 +427,6 @@ def test_latent_attention_cores_plan_is_a_function_of_the_shape():
     ops = _ops()
     assert ops.latent_attention_cores_plan(2048, 1, 12, 1024, 256) == (4, 0, 1)          # a prompt fills the chip uncut
     waves, keys, chunks = ops.latent_attention_cores_plan(8, 8, 12, 1024, 256)           # decoded tokens: cut
-    assert waves == 1 and keys == 128 and chunks * keys >= 1024 + 3
+    assert waves == 1 and keys == ops.mixing.LATENT_CHUNK_KEYS and chunks * keys >= 1024 + 3
     assert ops.latent_attention_cores_plan(8, 8, 12, 0, 256) == (1, 0, 1)                # no window, no cut
     assert ops.latent_attention_cores_plan(8, 8, 12, 72, 256) == (1, 0, 1)               # a window of one chunk

@@ -4,7 +4,10 @@
 // the keys its rows see in blocks of 32:
 //
 //   stage    the block's latents and key parts, [32][rank + rot], from the pages into LDS, rows padded by 16
-//            bytes; the latents once more transposed, [rank][32], for the second product
+//            bytes; the latents once more transposed, [rank][32], for the second product.  Neighbouring lanes take
+//            neighbouring keys, so that the transposed copy's 2-byte stores fall into neighbouring LDS banks (with
+//            neighbouring pieces of one key a lane, all 64 stores of an instruction met in one bank: 694 against
+//            381 us for a layer's 2,048 tokens)
 //   scores   S[key][row] = K . Q^T   v_mfma_f32_16x16x32_bf16: first operand the keys' rows from LDS, second the
 //            queries, held in registers for the whole walk (KS operands a lane)
 //   softmax  a lane holds 8 of a row's 32 scores, the row's other 24 are in 3 lanes: two lane exchanges; running
@@ -112,7 +115,7 @@ latent_attention_cores_kernel(float* __restrict__ out, float* __restrict__ parti
 #pragma unroll
             for (int u = 0; u < LA_BATCH; ++u) {
                 const int i = i0 + u * WAVES * ZI_WAVE;
-                const int key = (i / G) % LA_BK, d = (i % G) * 8, kp = kb + key;
+                const int key = i % LA_BK, d = ((i / LA_BK) % G) * 8, kp = kb + key;      // neighbouring lanes, neighbouring keys
                 // addresses are clamped, not guarded (a load under a branch would make every load before it
                 // wait), and what was read for a place that does not exist is masked
                 const bool want = i < LA_BK * G && kp <= k_hi && d < qw;
@@ -129,7 +132,7 @@ latent_attention_cores_kernel(float* __restrict__ out, float* __restrict__ parti
             for (int u = 0; u < LA_BATCH; ++u) {
                 const int i = i0 + u * WAVES * ZI_WAVE;
                 if (i >= LA_BK * G) break;
-                const int key = i / G, d = (i % G) * 8;
+                const int key = i % LA_BK, d = (i / LA_BK) * 8;
                 *reinterpret_cast<la_u32x4_t*>(&krow[key * KP + d]) = val[u].u;
                 if (d < RD) {
                     const unsigned keep = d < rank ? 0xffffffffu : 0u;      // the key parts are no values

@@ -210,7 +210,7 @@ union moe_pack {
     moe_bf16x8_t b;
 };
 
-template <typename TO, int RT>
+template <typename TO, int RT, int CT>      // a wavefront makes RT tiles of 16 rows x CT tiles of 16 columns
 __global__ void __launch_bounds__(256)
 moe_linear_mfma_kernel(TO* __restrict__ out, int64_t ldo, const zi_bf16* __restrict__ x, int64_t ldx,
                        const zi_bf16* __restrict__ w, const int32_t* __restrict__ plan,
@@ -220,41 +220,53 @@ moe_linear_mfma_kernel(TO* __restrict__ out, int64_t ldo, const zi_bf16* __restr
     const int e = plan[1 + 3 * tile], r0 = plan[2 + 3 * tile], rows = plan[3 + 3 * tile];
     const int lane = threadIdx.x % ZI_WAVE, wave = threadIdx.x / ZI_WAVE;
     const int r = lane % 16, j = lane / 16;
-    const int n0 = blockIdx.x * MOE_TN + wave * 16;
+    const int n0 = (blockIdx.x * 4 + wave) * 16 * CT;
     if (n0 >= N) return;
-    const int wn = n0 + r < N ? n0 + r : N - 1;
-    const zi_bf16* wrow = w + ((int64_t)e * N + wn) * K;
+    const zi_bf16* wrow[CT];
+#pragma unroll
+    for (int c = 0; c < CT; ++c) {
+        const int wn = n0 + 16 * c + r < N ? n0 + 16 * c + r : N - 1;
+        wrow[c] = w + ((int64_t)e * N + wn) * K;
+    }
     const zi_bf16* xrow[RT];
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
         const int rr = t * 16 + r < rows ? t * 16 + r : 0;
         xrow[t] = x + (int64_t)(source ? source[r0 + rr] / source_div : r0 + rr) * ldx;
     }
-    moe_f32x4_t acc[RT];
+    moe_f32x4_t acc[RT][CT];
 #pragma unroll
-    for (int t = 0; t < RT; ++t) acc[t] = (moe_f32x4_t){0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
+    for (int t = 0; t < RT; ++t)
+#pragma unroll
+        for (int c = 0; c < CT; ++c) acc[t][c] = (moe_f32x4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
     for (int k0 = 0; k0 < K; k0 += 32) {
         const int k = k0 + 8 * j;
         const bool in = k < K;      // K is a multiple of 8: a piece of eight lies inside or outside
         const int kc = in ? k : 0;
         const unsigned mask = 0u - (unsigned)in;
-        moe_pack a, b[RT];
-        a.u = *reinterpret_cast<const moe_u32x4_t*>(wrow + kc) & mask;
+        moe_pack a[CT], b[RT];
+#pragma unroll
+        for (int c = 0; c < CT; ++c) a[c].u = *reinterpret_cast<const moe_u32x4_t*>(wrow[c] + kc) & mask;
 #pragma unroll
         for (int t = 0; t < RT; ++t) b[t].u = *reinterpret_cast<const moe_u32x4_t*>(xrow[t] + kc) & mask;
 #pragma unroll
-        for (int t = 0; t < RT; ++t) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.b, b[t].b, acc[t], 0, 0, 0);
+        for (int t = 0; t < RT; ++t)
+#pragma unroll
+            for (int c = 0; c < CT; ++c)
+                acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[c].b, b[t].b, acc[t][c], 0, 0, 0);
     }
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
         const int row = t * 16 + r;
         if (row >= rows) continue;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const int n = n0 + 4 * j + i;
-            if (n < N) zi_store(out + (int64_t)(r0 + row) * ldo + n, moe_act(acc[t][i], act));
-        }
+        for (int c = 0; c < CT; ++c)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int n = n0 + 16 * c + 4 * j + i;
+                if (n < N) zi_store(out + (int64_t)(r0 + row) * ldo + n, moe_act(acc[t][c][i], act));
+            }
     }
 }
 
@@ -268,14 +280,16 @@ extern "C" int zi_moe_linear(void* out, int out_dt, int64_t ldo, const void* x, 
     const dim3 grid((N + MOE_TN - 1) / MOE_TN, max_tiles);
     const bool cores = x_dt == ZI_BF16 && w_dt == ZI_BF16 && K % 8 == 0 && ldx % 8 == 0 && ((uintptr_t)x % 16) == 0 &&
                        ((uintptr_t)w % 16) == 0 && (tile_rows == 16 || tile_rows == 32 || tile_rows == 64);
-#define ZI_MOE_CORES(RT)                                                                                        \
-    moe_linear_mfma_kernel<TO, RT><<<grid, 256, 0, stream>>>((TO*)out, ldo, (const zi_bf16*)x, ldx,              \
-                                                             (const zi_bf16*)w, plan, source, source_div, N, K, act)
+    // tiles of 64 rows (many rows an expert: prompts): a wavefront makes 64 columns of them, so that an operand of
+    // the tokens serves four of the weights'; smaller tiles (decoded tokens) are bound by the weights' stream
+#define ZI_MOE_CORES(RT, CT)                                                                                       \
+    moe_linear_mfma_kernel<TO, RT, CT><<<dim3((N + 64 * CT - 1) / (64 * CT), max_tiles), 256, 0, stream>>>(         \
+        (TO*)out, ldo, (const zi_bf16*)x, ldx, (const zi_bf16*)w, plan, source, source_div, N, K, act)
     if (cores) {
         ZI_DISPATCH_DTYPE(out_dt, TO, {
-            if (tile_rows == 16) ZI_MOE_CORES(1);
-            else if (tile_rows == 32) ZI_MOE_CORES(2);
-            else ZI_MOE_CORES(4);
+            if (tile_rows == 16) ZI_MOE_CORES(1, 1);
+            else if (tile_rows == 32) ZI_MOE_CORES(2, 2);
+            else ZI_MOE_CORES(4, 4);
         });
         return zi_check_launch("moe_linear");
     }

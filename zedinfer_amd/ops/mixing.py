@@ -3,6 +3,7 @@ latent attention (a short latent and one shared rotated key part per token), the
 matrix state per head), routed experts, and the gated activation in its other forms."""
 from __future__ import annotations
 
+import os
 from typing import Optional
 
 import torch
@@ -142,7 +143,8 @@ def latent_attention(qa: torch.Tensor, c_cache: torch.Tensor, kr_cache: torch.Te
     return out
 
 
-LATENT_CHUNK_KEYS = 128      # keys of a chunk when a tile's keys are cut over workgroups
+# keys of a chunk when a tile's keys are cut over workgroups (a multiple of the kernel's block of 32)
+LATENT_CHUNK_KEYS = max(32, int(os.environ.get("ZEDINFER_LATENT_CHUNK_KEYS", "128") or 128) // 32 * 32)
 
 
 def latent_attention_cores_supported(cache_dtype: torch.dtype, rank: int, rot: int) -> bool:
