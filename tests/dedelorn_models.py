@@ -115,3 +115,44 @@ def write_model(folder, name, seed=0, dtype=torch.float32):
         json.dump(cfg, f, indent=1)
     write_safetensors(os.path.join(folder, "model.safetensors"), make_weights(cfg, seed, dtype), metadata={"format": "pt"})
     return folder
+
+
+def random_config(seed):
+    """A configuration drawn at random: sizes, head counts, the order of layers, windows (from 1 key to more than a
+    sequence), which layers read whose latents, rotation bases, taps, experts and how many are chosen, norm eps."""
+    import random
+    rng = random.Random(seed)
+    width = rng.choice([48, 64, 96, 128, 160])
+    cfg = dict(architecture="Dedelorn", width=width, vocab=rng.choice([97, 256, 411]), norm=dict(eps=rng.choice([1e-6, 1e-5, 3e-6])),
+               layers=[])
+    owners = []                  # latent layers that keep a cache of their own
+    for i in range(rng.randint(2, 6)):
+        if rng.random() < 0.5:
+            kvh = rng.choice([1, 2, 3])
+            mixer = dict(heads=kvh * rng.choice([1, 2, 4]), kv_heads=kvh, dim=rng.choice([8, 16, 24, 40, 64, 96]),
+                         vdim=rng.choice([8, 16, 24, 40, 64]), conv=rng.choice([1, 2, 3, 4, 6]))
+            kind = "delta"
+        else:
+            kind = "latent_attention"
+            if owners and rng.random() < 0.5:
+                src = rng.choice(owners)
+                o = cfg["layers"][src]["mixer"]
+                mixer = dict(kv_rank=o["kv_rank"], rot_dim=o["rot_dim"], rot=dict(o["rot"]), kv_from=src)
+            else:
+                rot = rng.choice([2, 4, 8, 16, 24, 32])
+                mixer = dict(kv_rank=rng.choice([16, 24, 40, 64, 96, 136]), rot_dim=rot,
+                             rot=dict(base=rng.choice([50.0, 10000.0, 500000.0]), dims=rot))
+                owners.append(i)
+            mixer.update(heads=rng.choice([1, 2, 3, 5, 8, 17]), dim=rng.choice([8, 16, 24, 32, 48]), vdim=rng.choice([8, 16, 24, 40]),
+                         scale=rng.choice([0.1, 0.25, 0.5]), mask=dict(size=rng.choice([1, 2, 7, 16, 31, 64, 100, 500])))
+        r = rng.random()
+        if r < 0.2:
+            mlp = None
+        elif r < 0.6:
+            mlp = dict(kind="dense", ff=rng.choice([32, 72, 136]))
+        else:
+            experts = rng.choice([2, 4, 7, 16, 40])
+            mlp = dict(kind="moe", expert=dict(ff=rng.choice([16, 40, 72])),
+                       router=dict(experts=experts, top=rng.randint(1, min(experts, 6)), scale=rng.choice([1.0, 2.5, 0.5])))
+        cfg["layers"].append(dict(type=kind, mixer=mixer, mlp=mlp))
+    return cfg

@@ -201,3 +201,31 @@ def test_command_lines_take_a_model_of_the_design(tmp_path):
     r = run(os.path.join(ROOT, "bin", "batch_bench"), str(tmp_path / "cfg"), "-b", "3", "-p", "20", "-d", "6", "--num-kv-blocks",
             "64", "--kv-block-size", "8", "--random-weights", "--seed", "4", "--no-log-to-console")
     assert r.returncode == 0 and "18 tokens generated" in r.stdout, r.stderr + r.stdout
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_configurations_drawn_at_random(tmp_path, seed):
+    """Twelve models whose sizes, layer order, windows, shared caches and constants are drawn at random, each in both
+    engine types, over a batch of unequal requests with pages and slots used again and over whole prompts."""
+    import json
+    from zedinfer_amd.config import SchedulerConfig
+    from zedinfer_amd.engine import Engine
+    from zedinfer_amd.weights.safetensors_io import write_safetensors
+    cfg = models.random_config(seed)
+    requests = {f"z{i}": traces.random_tokens(cfg["vocab"], n, seed=seed * 10 + i) for i, n in enumerate([83, 5, 140, 31, 1, 66])}
+    for dtype in ("float32", "bfloat16"):
+        folder = str(tmp_path / dtype)
+        os.makedirs(folder)
+        with open(os.path.join(folder, "config.json"), "w") as f:
+            json.dump(cfg, f)
+        write_safetensors(os.path.join(folder, "model.safetensors"),
+                          models.make_weights(cfg, seed, torch.float32 if dtype == "float32" else torch.bfloat16), metadata={"format": "pt"})
+        pcfg, w = plain.load_folder(folder, torch.float64)
+        ref = {rid: plain.forward(pcfg, w, toks).float() for rid, toks in requests.items()}
+        ps = [4, 8, 16, 32][seed % 4]
+        engine = Engine.from_folder(folder, dtype, SchedulerConfig(num_kv_blocks=3 * -(-140 // ps) + 6, kv_block_size=ps,
+                                                                   max_batch_requests=3, max_batch_tokens=4096, max_seq_len=4096))
+        for what, steps in (("mixed", traces.mixed(requests, max_live=3, seed=seed, decode_tail=25, max_portion=40)),
+                            ("whole", traces.whole(requests))):
+            out = traces.run_in_process(engine, steps)
+            _check(steps, out, ref, requests, dtype, (what, seed, json.dumps(cfg)))
