@@ -280,3 +280,104 @@ class DedelornConfig(ModelConfig):
         if self.eos_token_ids:
             d["eos_token_id"] = list(self.eos_token_ids)
         return d
+
+
+@dataclass(frozen=True)
+class TosisunConfig(ModelConfig):
+    """The Tosisun design's config.json: ``width``, ``vocab``, ``norm.eps``, ``logit_softcap`` (optional) and a list
+    ``layers`` whose entries each name a mixer by ``type`` ("attention": grouped-query attention whose projections
+    pass a short convolution, with a sink in the softmax) with its sizes under ``mixer`` and a feed-forward under
+    ``mlp`` (``kind`` "dense" or "moe", or null for none).  An entry with ``weights_of``: j runs with layer j's
+    tensors and a cache and state of its own.  Every size and constant of a model is read from here; the shared keys
+    of ``ModelConfig`` that the format does not have keep their neutral values."""
+
+    layers: Tuple[Any, ...] = ()
+    norm_eps: float = 1e-5
+    logit_softcap: float = 0.0
+
+    MIXER_KEYS = {"attention": ("heads", "kv_heads", "dim", "vdim", "conv", "scale", "rot")}
+
+    @classmethod
+    def from_dict(cls, d: Mapping[str, Any]) -> "TosisunConfig":
+        missing = [k for k in ("width", "vocab", "layers", "norm") if k not in d]
+        if missing:
+            raise ConfigError("config.json lacks required key(s): " + ", ".join(missing))
+        if not isinstance(d["layers"], (list, tuple)) or not d["layers"]:
+            raise ConfigError("config.json: 'layers' must be a non-empty list")
+        if not isinstance(d["norm"], Mapping) or "eps" not in d["norm"]:
+            raise ConfigError("config.json: 'norm' must give 'eps'")
+        eos = d.get("eos_token_id")
+        cap = d.get("logit_softcap")
+        cfg = cls(architectures=(str(d.get("architecture", "Tosisun")),), model_type="tosisun",
+                  torch_dtype=str(d.get("torch_dtype") or "bfloat16"), hidden_size=_as_int(d, "width"),
+                  vocab_size=_as_int(d, "vocab"), num_hidden_layers=len(d["layers"]),
+                  eos_token_ids=() if eos is None else tuple(int(e) for e in (eos if isinstance(eos, (list, tuple)) else [eos])),
+                  layers=tuple(json.loads(json.dumps(layer)) for layer in d["layers"]), norm_eps=float(d["norm"]["eps"]),
+                  logit_softcap=float(cap) if cap else 0.0)
+        cfg.validate()
+        return cfg
+
+    def validate(self) -> None:
+        if self.hidden_size <= 0 or self.vocab_size <= 0:
+            raise ConfigError("config.json: 'width' and 'vocab' must be positive")
+        if not (self.norm_eps > 0):
+            raise ConfigError(f"config.json: norm.eps must be positive, got {self.norm_eps}")
+        if self.logit_softcap < 0:
+            raise ConfigError(f"config.json: logit_softcap must be positive, got {self.logit_softcap}")
+        for i, layer in enumerate(self.layers):
+            kind = layer.get("type") if isinstance(layer, Mapping) else None
+            if kind not in self.MIXER_KEYS:
+                raise ConfigError(f"config.json: layer {i} has type {kind!r}; known: {', '.join(sorted(self.MIXER_KEYS))}")
+            src = layer.get("weights_of")
+            if src is not None:
+                ok = isinstance(src, int) and not isinstance(src, bool) and 0 <= src < i \
+                    and self.layers[src].get("weights_of") is None
+                if not ok:
+                    raise ConfigError(f"config.json: layer {i}: weights_of must name an earlier layer with tensors of its own")
+                o = self.layers[src]
+                if (o.get("type"), o.get("mixer"), o.get("mlp")) != (layer.get("type"), layer.get("mixer"), layer.get("mlp")):
+                    raise ConfigError(f"config.json: layer {i}: a layer that uses layer {src}'s weights must equal it in "
+                                      "type, mixer and mlp")
+            m = layer.get("mixer")
+            lacking = [k for k in self.MIXER_KEYS[kind] if not isinstance(m, Mapping) or k not in m]
+            if lacking:
+                raise ConfigError(f"config.json: layer {i} ({kind}) lacks mixer key(s): " + ", ".join(lacking))
+            if any(int(m[k]) <= 0 for k in ("heads", "kv_heads", "dim", "vdim", "conv")) or int(m["heads"]) % int(m["kv_heads"]):
+                raise ConfigError(f"config.json: layer {i}: heads, kv_heads, dim, vdim and conv must be positive, heads a "
+                                  "multiple of kv_heads")
+            if not float(m["scale"]) > 0:
+                raise ConfigError(f"config.json: layer {i}: scale must be positive")
+            rot = m["rot"]
+            if not isinstance(rot, Mapping) or int(rot.get("dims", -1)) < 0 or int(rot.get("dims", -1)) % 2 \
+                    or int(rot["dims"]) > int(m["dim"]) or (int(rot["dims"]) > 0 and not float(rot.get("base", 0)) > 0):
+                raise ConfigError(f"config.json: layer {i}: rot.dims must be even and within dim, rot.base positive")
+            sc = rot.get("scaling")
+            if sc is not None and (not isinstance(sc, Mapping) or any(k not in sc for k in ("factor", "low", "high", "original"))):
+                raise ConfigError(f"config.json: layer {i}: rot.scaling needs factor, low, high and original")
+            mlp = layer.get("mlp")
+            if mlp is None:
+                continue
+            if mlp.get("kind") == "dense":
+                if not int(mlp.get("ff", 0)) > 0:
+                    raise ConfigError(f"config.json: layer {i}: a dense mlp needs a positive 'ff'")
+            elif mlp.get("kind") == "moe":
+                r, ex = mlp.get("router") or {}, mlp.get("expert") or {}
+                if not int(ex.get("ff", 0)) > 0 or not float(ex.get("limit", 0)) > 0 \
+                        or not (0 < int(r.get("top", 0)) <= int(r.get("experts", 0))):
+                    raise ConfigError(f"config.json: layer {i}: a moe mlp needs expert.ff, expert.limit, router.experts and "
+                                      "router.top (at most the experts)")
+                sh = mlp.get("shared")
+                if sh is not None and (not int(sh.get("ff", 0)) > 0 or not float(sh.get("limit", 0)) > 0):
+                    raise ConfigError(f"config.json: layer {i}: a shared expert needs ff and limit")
+            else:
+                raise ConfigError(f"config.json: layer {i}: mlp.kind {mlp.get('kind')!r} is neither 'dense' nor 'moe'")
+
+    def to_dict(self) -> Dict[str, Any]:
+        d = {"architecture": self.architectures[0] if self.architectures else "Tosisun",
+             "layers": json.loads(json.dumps(list(self.layers))), "norm": {"eps": self.norm_eps},
+             "vocab": self.vocab_size, "width": self.hidden_size}
+        if self.logit_softcap:
+            d["logit_softcap"] = self.logit_softcap
+        if self.eos_token_ids:
+            d["eos_token_id"] = list(self.eos_token_ids)
+        return d

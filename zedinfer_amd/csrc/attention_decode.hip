@@ -76,7 +76,7 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
                         const int32_t* __restrict__ tok_index, const int32_t* __restrict__ tok_seq,
                         const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_tables,
                         int max_pages, int num_pages, int nh, int nkv, int G, int ps, int window, float scale,
-                        int max_chunks, int leave_parts, DecProjection pj) {
+                        int max_chunks, int leave_parts, DecProjection pj, const float* __restrict__ sinks) {
     static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
     constexpr int DK = (D + 31) / 32;   // k-steps of the score product
     constexpr int DT = D / 16;          // output tiles of 16 dims
@@ -512,7 +512,9 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
         L += a[w] * sl[w][r];
     }
     const bool final = sp.count == 1 && !leave_parts;
-    const float inv = final ? 1.f / L : 1.f;
+    // a sink counts once in the denominator, as exp(sink) (maxima are in base-2 units)
+    const float sink_w = (final && sinks && r < G) ? __builtin_amdgcn_exp2f(sinks[kvh * G + r] * 1.4426950408889634f - M) : 0.f;
+    const float inv = final ? 1.f / (L + sink_w) : 1.f;
     const int64_t slot = zi_dec_part_slot(x, nh, kvh * G + r, chunk);
     for (int dd = wave; dd < DT; dd += DEC_WAVES) {
         dec_f32x4_t acc = dec_f32x4_t{0.f, 0.f, 0.f, 0.f};
@@ -541,7 +543,8 @@ attention_decode_kernel(zi_bf16* __restrict__ out, int64_t ldo, float* __restric
 __global__ void __launch_bounds__(ZI_WAVE)
 attention_decode_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const float* __restrict__ part_o,
                               const float* __restrict__ part_ml, const int32_t* __restrict__ tok_index,
-                              const int32_t* __restrict__ tok_pos, int nh, int D, int window, int max_chunks) {
+                              const int32_t* __restrict__ tok_pos, int nh, int D, int window, int max_chunks,
+                              const float* __restrict__ sinks) {
     const int x = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int t = tok_index ? tok_index[x] : x;
     const DecSplit sp = dec_split(tok_pos[t], window);
@@ -569,6 +572,7 @@ attention_decode_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const floa
             acc[1] += w * po[c][1];
         }
     }
+    if (sinks) L += __builtin_amdgcn_exp2f(sinks[h] * 1.4426950408889634f - M);
     const float inv = 1.f / L;
 #pragma unroll
     for (int v = 0; v < 2; ++v)
@@ -731,7 +735,7 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
                       const void* kcache, const void* vcache, const int32_t* tok_index, const int32_t* tok_seq,
                       const int32_t* tok_pos, const int32_t* block_tables, int max_pages, int num_pages, int nh, int nkv,
                       int d, int page_size, int window, float scale, int max_chunks, float* workspace,
-                      int64_t workspace_floats, const DecProjection* pj, hipStream_t stream) {
+                      int64_t workspace_floats, const DecProjection* pj, const float* sinks, hipStream_t stream) {
     ZI_REQUIRE(zi_attention_decode_supported(dt, nh, nkv, d, page_size),
                "%s: unsupported shape (bfloat16, head_dim a multiple of 16 up to 128, group <= 16, "
                "page size %% 8 == 0): dtype %d heads %d kv_heads %d head_dim %d page %d", who, dt, nh, nkv, d, page_size);
@@ -760,12 +764,12 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
         attention_decode_kernel<DD, true, VMODE><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                 \
             (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
             tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
-            max_chunks, leave_parts, *pj);                                                                                      \
+            max_chunks, leave_parts, *pj, sinks);                                                                                      \
     else                                                                                                             \
         attention_decode_kernel<DD, false, VMODE><<<grid, DEC_WAVES * ZI_WAVE, 0, stream>>>(                                \
             (zi_bf16*)out, ldo, po, pml, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache,     \
             tok_index, tok_seq, tok_pos, block_tables, max_pages, num_pages, nh, nkv, G, page_size, window, scale,   \
-            max_chunks, leave_parts, none)
+            max_chunks, leave_parts, none, sinks)
     switch (d) {
         case 16: ZI_DEC(16, 0); break;
         case 32: ZI_DEC(32, 0); break;
@@ -783,7 +787,7 @@ static int dec_launch(const char* who, void* out, const void* q, int dt, int n_i
 #undef ZI_DEC
     if (max_chunks > 1 && !leave_parts)
         attention_decode_merge_kernel<<<dim3(n_idx, nh), ZI_WAVE, 0, stream>>>((zi_bf16*)out, ldo, po, pml, tok_index,
-                                                                              tok_pos, nh, d, window, max_chunks);
+                                                                              tok_pos, nh, d, window, max_chunks, sinks);
     return zi_check_launch(who);
 }
 
@@ -795,7 +799,21 @@ extern "C" int zi_attention_decode(void* out, const void* q, int dt, int n_idx, 
                                    hipStream_t stream) {
     return dec_launch("attention_decode", out, q, dt, n_idx, ldq, ldo, kcache, vcache, tok_index, tok_seq, tok_pos,
                       block_tables, max_pages, num_pages, nh, nkv, d, page_size, window, scale, max_chunks, workspace,
-                      workspace_floats, nullptr, stream);
+                      workspace_floats, nullptr, nullptr, stream);
+}
+
+// The same with `sinks` (float32 [nh]): the softmax of head h also counts exp(sinks[h]) in its denominator, once,
+// whatever the number of chunks a token's keys are cut into.
+extern "C" int zi_attention_decode_sink(void* out, const void* q, int dt, int n_idx, int64_t ldq, int64_t ldo,
+                                        const void* kcache, const void* vcache, const int32_t* tok_index,
+                                        const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables,
+                                        int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
+                                        float scale, int max_chunks, float* workspace, int64_t workspace_floats,
+                                        const float* sinks, hipStream_t stream) {
+    ZI_REQUIRE(out != nullptr, "attention_decode_sink: the chunks cannot be left unmerged");
+    return dec_launch("attention_decode_sink", out, q, dt, n_idx, ldq, ldo, kcache, vcache, tok_index, tok_seq, tok_pos,
+                      block_tables, max_pages, num_pages, nh, nkv, d, page_size, window, scale, max_chunks, workspace,
+                      workspace_floats, nullptr, sinks, stream);
 }
 
 // 1 when the fused entry point takes this projection layout, else 0 (then: rotate and store first, and
@@ -841,7 +859,7 @@ extern "C" int zi_attention_decode_fused(void* out, int dt, int n_idx, int64_t l
     pj.table = table; pj.rot = rot; pj.slots = slots; pj.cache_slots = cache_slots; pj.write_kv = write_kv;
     return dec_launch("attention_decode_fused", out, nullptr, dt, n_idx, 0, ldo, kcache, vcache, tok_index, tok_seq,
                       tok_pos, block_tables, max_pages, num_pages, nh, nkv, d, page_size, window, scale, max_chunks,
-                      workspace, workspace_floats, &pj, stream);
+                      workspace, workspace_floats, &pj, nullptr, stream);
 }
 
 // Heads whose merged attention one workgroup of the projection multiplies (one partial sum for each

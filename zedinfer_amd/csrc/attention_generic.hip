@@ -27,7 +27,7 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
                          const int32_t* __restrict__ tok_index, const int32_t* __restrict__ tok_seq,
                          const int32_t* __restrict__ tok_pos, const int32_t* __restrict__ block_tables,
                          int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
-                         float scale) {
+                         float scale, const float* __restrict__ sinks) {
     __shared__ float qs[ATTN_MAX_D];
     __shared__ float ps[ZI_WAVE];
     __shared__ int64_t vbase[ZI_WAVE];
@@ -90,6 +90,8 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
         __syncthreads();
     }
     T* orow = out + (int64_t)t * ldo + (int64_t)h * d;
+    // a sink counts once in the denominator: exp(sink), unscaled, with no key and no value
+    if (sinks) l += expf(sinks[h] - m);
     const float inv = 1.f / l;
 #pragma unroll
     for (int i = 0; i < ATTN_ACC; ++i) {
@@ -98,11 +100,12 @@ attention_generic_kernel(T* __restrict__ out, const T* __restrict__ q, int64_t l
     }
 }
 
-extern "C" int zi_attention_generic(void* out, const void* q, int dt, int n, int64_t ldq, int64_t ldo,
-                                    const void* kcache, const void* vcache, const int32_t* tok_index,
-                                    const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables, int max_pages,
-                                    int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
-                                    hipStream_t stream) {
+// `sinks` (float32 [nh], or null): the softmax of head h also counts exp(sinks[h]) in its denominator.
+extern "C" int zi_attention_generic_sink(void* out, const void* q, int dt, int n, int64_t ldq, int64_t ldo,
+                                         const void* kcache, const void* vcache, const int32_t* tok_index,
+                                         const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables,
+                                         int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
+                                         float scale, const float* sinks, hipStream_t stream) {
     ZI_REQUIRE(n >= 0 && nh > 0 && nkv > 0 && d > 0 && page_size > 0 && max_pages > 0 && num_pages > 0,
                "attention: bad sizes");
     ZI_REQUIRE(nh % nkv == 0, "attention: %d query heads are not a multiple of %d key/value heads", nh, nkv);
@@ -114,7 +117,16 @@ extern "C" int zi_attention_generic(void* out, const void* q, int dt, int n, int
     ZI_DISPATCH_DTYPE(dt, T, {
         attention_generic_kernel<T><<<dim3(n, nh), ZI_WAVE, 0, stream>>>(
             (T*)out, (const T*)q, ldq, ldo, (const T*)kcache, (const T*)vcache, tok_index, tok_seq, tok_pos, block_tables,
-            max_pages, num_pages, nh, nkv, d, page_size, window, scale);
+            max_pages, num_pages, nh, nkv, d, page_size, window, scale, sinks);
     });
     return zi_check_launch("attention_generic");
+}
+
+extern "C" int zi_attention_generic(void* out, const void* q, int dt, int n, int64_t ldq, int64_t ldo,
+                                    const void* kcache, const void* vcache, const int32_t* tok_index,
+                                    const int32_t* tok_seq, const int32_t* tok_pos, const int32_t* block_tables, int max_pages,
+                                    int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
+                                    hipStream_t stream) {
+    return zi_attention_generic_sink(out, q, dt, n, ldq, ldo, kcache, vcache, tok_index, tok_seq, tok_pos, block_tables,
+                                     max_pages, num_pages, nh, nkv, d, page_size, window, scale, nullptr, stream);
 }

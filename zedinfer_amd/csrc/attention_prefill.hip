@@ -69,7 +69,8 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
                          const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
                          const int32_t* __restrict__ entry_past, const int32_t* __restrict__ block_tables,
                          int max_pages, int num_pages, int nh, int nkv, int ps_shift, int window, float scale,
-                         float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks, int chunk_keys) {
+                         float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks, int chunk_keys,
+                         const float* __restrict__ sinks) {
     static_assert(D % 16 == 0 && D >= 16 && D <= 128, "head_dim must be a multiple of 16 up to 128");
     constexpr int DK = (D + 31) / 32;   // k-steps of the score product
     constexpr int DP = DK * 32;         // head_dim padded to a multiple of 32
@@ -378,6 +379,8 @@ attention_prefill_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf16* 
         }
         return;
     }
+    // a sink counts once in the denominator, as exp(sink) (the maximum is in base-2 units)
+    if (sinks) l += __builtin_amdgcn_exp2f(sinks[h] * 1.4426950408889634f - m);
     const float inv = 1.f / l;
     zi_bf16* orow = out + (int64_t)(start + off + row) * ldo + (int64_t)h * D;
 #pragma unroll
@@ -421,7 +424,8 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
                              const int32_t* __restrict__ entry_start, const int32_t* __restrict__ entry_len,
                              const int32_t* __restrict__ entry_past, const int32_t* __restrict__ block_tables,
                              int max_pages, int num_pages, int nh, int nkv, int ps_shift, int window, float scale,
-                             float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks, int chunk_keys) {
+                             float* __restrict__ part_o, float* __restrict__ part_ml, int max_chunks, int chunk_keys,
+                             const float* __restrict__ sinks) {
     static_assert(D == 64 || D == 128, "this variant takes head sizes 64 and 128");
     static_assert(QW == 1 || QW == 2, "16 or 32 queries a wavefront");
     constexpr int BM = PF_BM * QW;                   // queries of a tile
@@ -728,7 +732,7 @@ attention_prefill_dma_kernel(zi_bf16* __restrict__ out, int64_t ldo, const zi_bf
             }
             continue;
         }
-        const float inv = 1.f / l[u];
+        const float inv = 1.f / (l[u] + (sinks ? __builtin_amdgcn_exp2f(sinks[h] * 1.4426950408889634f - m[u]) : 0.f));
         zi_bf16* orow = out + (int64_t)(start + off + row[u]) * ldo + (int64_t)h * D;
 #pragma unroll
         for (int dd = 0; dd < DT; ++dd) {
@@ -747,7 +751,8 @@ attention_prefill_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const flo
                                const float* __restrict__ part_ml, const int32_t* __restrict__ tile_entry,
                                const int32_t* __restrict__ tile_off, const int32_t* __restrict__ entry_start,
                                const int32_t* __restrict__ entry_len, const int32_t* __restrict__ entry_past, int nh,
-                               int D, int window, int max_chunks, int bm, int chunk_keys) {
+                               int D, int window, int max_chunks, int bm, int chunk_keys,
+                               const float* __restrict__ sinks) {
     const int tile = blockIdx.x / bm, qi = blockIdx.x % bm, h = blockIdx.y, lane = threadIdx.x;
     const int e = tile_entry[tile], off = tile_off[tile];
     const int start = entry_start[e], len = entry_len[e], past = entry_past[e];
@@ -770,6 +775,7 @@ attention_prefill_merge_kernel(zi_bf16* __restrict__ out, int64_t ldo, const flo
         for (int v = 0; v < 2; ++v)
             if (lane + v * ZI_WAVE < D) acc[v] += w * part_o[(slot0 + c) * D + lane + v * ZI_WAVE];
     }
+    if (sinks) L += __builtin_amdgcn_exp2f(sinks[h] * 1.4426950408889634f - M);
     const float inv = 1.f / L;
 #pragma unroll
     for (int v = 0; v < 2; ++v)
@@ -842,13 +848,15 @@ extern "C" int zi_attention_prefill_cuts(int max_keys, int window, int groups, i
 // position entry_past[e] of its sequence, whose block table is row e of block_tables.  `alone` (head sizes 64 and
 // 128): workgroups of four wavefronts that walk blocks of 64 keys, two to a compute unit, for launches of many
 // tiles; a query's keys are then added in another order, so the result differs by rounding.
-extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,
-                                    const void* kcache, const void* vcache, const int32_t* tile_entry,
-                                    const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
-                                    const int32_t* entry_past, const int32_t* block_tables, int max_pages,
-                                    int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
-                                    int rows, int max_chunks, float* workspace, int64_t workspace_floats, int tile,
-                                    int alone, int chunk_keys, hipStream_t stream) {
+// `sinks` (float32 [nh], or null): the softmax of head h also counts exp(sinks[h]) in its denominator, once, whatever
+// the number of cuts of a tile's keys.
+extern "C" int zi_attention_prefill_sink(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,
+                                         const void* kcache, const void* vcache, const int32_t* tile_entry,
+                                         const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
+                                         const int32_t* entry_past, const int32_t* block_tables, int max_pages,
+                                         int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
+                                         int rows, int max_chunks, float* workspace, int64_t workspace_floats, int tile,
+                                         int alone, int chunk_keys, const float* sinks, hipStream_t stream) {
     ZI_REQUIRE(tile == PF_BM || (tile == 2 * PF_BM && pf_variant >= 1 && (d == 64 || d == 128)),
                "attention_prefill: tiles of %d queries (64, or 128 for head sizes 64 and 128)", tile);
     ZI_REQUIRE(zi_attention_prefill_supported(dt, nh, nkv, d, page_size),
@@ -880,12 +888,12 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
     attention_prefill_kernel<DD><<<grid, PF_WAVES * ZI_WAVE, 0, stream>>>(                                     \
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
         tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
-        window, scale, po, pml, max_chunks, chunk_keys)
+        window, scale, po, pml, max_chunks, chunk_keys, sinks)
 #define ZI_PF_DMA(DD, QW, KH)                                                                                  \
     attention_prefill_dma_kernel<DD, QW, KH><<<grid, 4 * KH * ZI_WAVE, 0, stream>>>(                           \
         (zi_bf16*)out, ldo, (const zi_bf16*)q, ldq, (const zi_bf16*)kcache, (const zi_bf16*)vcache, tile_entry, \
         tile_off, entry_start, entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, ps_shift,   \
-        window, scale, po, pml, max_chunks, chunk_keys)
+        window, scale, po, pml, max_chunks, chunk_keys, sinks)
     const bool dma = pf_variant >= 1 && (d == 64 || d == 128);
     const bool wide = tile == 2 * PF_BM;
     ZI_REQUIRE(!alone || dma, "attention_prefill: workgroups of four wavefronts are for head sizes 64 and 128");
@@ -913,6 +921,19 @@ extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_ti
     if (max_chunks > 1)
         attention_prefill_merge_kernel<<<dim3(num_tiles * tile, nh), ZI_WAVE, 0, stream>>>(
             (zi_bf16*)out, ldo, po, pml, tile_entry, tile_off, entry_start, entry_len, entry_past, nh, d, window, max_chunks,
-            tile, chunk_keys);
+            tile, chunk_keys, sinks);
     return zi_check_launch("attention_prefill");
+}
+
+extern "C" int zi_attention_prefill(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo,
+                                    const void* kcache, const void* vcache, const int32_t* tile_entry,
+                                    const int32_t* tile_off, const int32_t* entry_start, const int32_t* entry_len,
+                                    const int32_t* entry_past, const int32_t* block_tables, int max_pages,
+                                    int num_pages, int nh, int nkv, int d, int page_size, int window, float scale,
+                                    int rows, int max_chunks, float* workspace, int64_t workspace_floats, int tile,
+                                    int alone, int chunk_keys, hipStream_t stream) {
+    return zi_attention_prefill_sink(out, q, dt, num_tiles, ldq, ldo, kcache, vcache, tile_entry, tile_off, entry_start,
+                                     entry_len, entry_past, block_tables, max_pages, num_pages, nh, nkv, d, page_size,
+                                     window, scale, rows, max_chunks, workspace, workspace_floats, tile, alone,
+                                     chunk_keys, nullptr, stream);
 }

@@ -1,0 +1,173 @@
+// What stands between the q/k/v projection and attention in a mixer whose projections pass a short causal
+// convolution over time: per token and in float32,
+//
+//   u = projection + bias                                             [q | k | v] channels, C in all
+//   y_t[c] = sum_j taps[c][j] * u_(t - (taps-1) + j)[c]                 zeros before the sequence's start
+//   q = y_q / rms(y_q) * w_q,  k = y_k / rms(y_k) * w_k                 one root mean square over ALL heads' channels
+//   the first R dims of every head of q and k turn in pairs (i, i + R/2) by the step's angles
+//   q -> q_out [n][heads * D];  k, v -> the paged cache at the token's slot (heads of D values; a head of fewer
+//   dims is followed by zeros, so that one head size serves keys of `dim` and values of `vdim` dims)
+//
+// Rows of the entry's earlier tokens in this step come from the projection itself, rows before the step from the
+// request's tail: the last taps - 1 rows of u (bias included), float32, [taps-1][C] in the request's state slot,
+// zero for a fresh request (`zi_conv_tail` writes the new tail after this kernel has read the old one).
+//
+// One workgroup per token; the convolved channels pass through LDS.  Sums run in an order fixed by the sizes.
+#include "zi_common.h"
+#include "zi_api.h"
+
+#define CQ_THREADS 256
+#define CQ_MAX_CHANNELS 15360
+#define CQ_MAX_TAPS 16
+
+template <typename TP>
+__device__ __forceinline__ float cq_conv(const TP* __restrict__ proj, int64_t ld, const float* __restrict__ bias,
+                                         const float* __restrict__ conv_w, const float* __restrict__ tail, int t,
+                                         int local, int c, int C, int taps) {
+    float y = 0.f;
+    const float bc = bias ? bias[c] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int li = local - (taps - 1) + j;
+        const float u = li >= 0 ? zi_load(proj + (int64_t)(t - local + li) * ld + c) + bc
+                                : tail[(int64_t)(li + taps - 1) * C + c];
+        y += conv_w[(int64_t)c * taps + j] * u;
+    }
+    return y;
+}
+
+template <typename TP, typename T>
+__global__ void __launch_bounds__(CQ_THREADS)
+conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* __restrict__ vcache,
+                const TP* __restrict__ proj, int64_t ld, const float* __restrict__ bias, const float* __restrict__ conv_w,
+                const float* __restrict__ state, int64_t state_stride, const float* __restrict__ q_norm,
+                const float* __restrict__ k_norm, float eps, const float* __restrict__ table, int rot,
+                const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ entry_start,
+                const int32_t* __restrict__ entry_slot, const int32_t* __restrict__ slots, int64_t cache_slots, int nh,
+                int nkv, int dim, int vdim, int D, int taps, int page_size) {
+    extern __shared__ float y[];      // [C]
+    __shared__ float red[16];
+    const int t = blockIdx.x, e = tok_seq[t], local = t - entry_start[e];
+    const int Qd = nh * dim, Kd = nkv * dim, Vd = nkv * vdim, C = Qd + Kd + Vd;
+    const float* tail = state + (int64_t)entry_slot[e] * state_stride;
+    float sq = 0.f, sk = 0.f;
+    for (int c = threadIdx.x; c < C; c += CQ_THREADS) {
+        const float v = cq_conv(proj, ld, bias, conv_w, tail, t, local, c, C, taps);
+        y[c] = v;
+        if (c < Qd) sq += v * v;
+        else if (c < Qd + Kd) sk += v * v;
+    }
+    sq = zi_block_sum(sq, red);
+    sk = zi_block_sum(sk, red);
+    __syncthreads();
+    const float rq = 1.f / sqrtf(sq / (float)Qd + eps), rk = 1.f / sqrtf(sk / (float)Kd + eps);
+    const int half = rot / 2;
+    const float* ang = table ? table + (int64_t)t * half * 2 : nullptr;
+    // queries: every (head, dim of the padded head)
+    for (int i = threadIdx.x; i < nh * D; i += CQ_THREADS) {
+        const int h = i / D, x = i % D;
+        float v = 0.f;
+        if (x < dim) {
+            const int c = h * dim + x;
+            v = y[c] * rq * q_norm[c];
+            if (x < rot) {
+                const int p = x < half ? x : x - half;
+                const float cs = ang[2 * p], sn = ang[2 * p + 1];
+                const int co = x < half ? c + half : c - half;
+                const float o = y[co] * rq * q_norm[co];
+                v = x < half ? v * cs - o * sn : v * cs + o * sn;
+            }
+        }
+        zi_store(q_out + (int64_t)t * ldq + i, v);
+    }
+    const int slot = slots ? slots[t] : -1;
+    if (slot < 0 || (int64_t)slot >= cache_slots) return;      // a token without a place in the cache stores nothing
+    const int64_t page = slot / page_size, off = slot % page_size;
+    for (int i = threadIdx.x; i < nkv * D; i += CQ_THREADS) {
+        const int g = i / D, x = i % D;
+        float v = 0.f;
+        if (x < dim) {
+            const int c = g * dim + x;
+            v = y[Qd + c] * rk * k_norm[c];
+            if (x < rot) {
+                const int p = x < half ? x : x - half;
+                const float cs = ang[2 * p], sn = ang[2 * p + 1];
+                const int co = x < half ? c + half : c - half;
+                const float o = y[Qd + co] * rk * k_norm[co];
+                v = x < half ? v * cs - o * sn : v * cs + o * sn;
+            }
+        }
+        zi_store(kcache + ((page * nkv + g) * page_size + off) * D + x, v);
+    }
+    for (int i = threadIdx.x; i < nkv * D; i += CQ_THREADS) {
+        const int g = i / D, x = i % D;
+        const float v = x < vdim ? y[Qd + Kd + g * vdim + x] : 0.f;
+        zi_store(vcache + ((page * nkv + g) * D + x) * page_size + off, v);
+    }
+}
+
+extern "C" int zi_conv_qkv(void* q_out, int dt, int64_t ldq, void* kcache, void* vcache, const void* proj, int proj_dt,
+                           int64_t ld, const float* bias, const float* conv_w, const float* state, int64_t state_stride,
+                           const float* q_norm, const float* k_norm, float eps, const float* table, int rot, int n,
+                           const int32_t* tok_seq, const int32_t* entry_start, const int32_t* entry_slot,
+                           const int32_t* slots, int64_t cache_slots, int nh, int nkv, int dim, int vdim, int D, int taps,
+                           int page_size, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && dim > 0 && vdim > 0 && D >= dim && D >= vdim && taps >= 1 &&
+                   taps <= CQ_MAX_TAPS && page_size > 0,
+               "conv_qkv: bad sizes (heads %d/%d, dim %d, vdim %d, head size %d, taps %d)", nh, nkv, dim, vdim, D, taps);
+    const int64_t C = (int64_t)nh * dim + (int64_t)nkv * dim + (int64_t)nkv * vdim;
+    ZI_REQUIRE(C <= CQ_MAX_CHANNELS, "conv_qkv: %lld channels are more than %d", (long long)C, CQ_MAX_CHANNELS);
+    ZI_REQUIRE(ld >= C && ldq >= (int64_t)nh * D, "conv_qkv: a row is too short");
+    ZI_REQUIRE(state_stride >= (int64_t)(taps - 1) * C, "conv_qkv: the state row is too short");
+    ZI_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dim && (rot == 0 || table), "conv_qkv: %d rotated dims of %d", rot, dim);
+    ZI_REQUIRE(eps > 0.f, "conv_qkv: eps must be positive");
+    ZI_REQUIRE(!slots || (kcache && vcache && cache_slots > 0), "conv_qkv: slots without a cache");
+    if (n == 0) return 0;
+    const size_t lds = (size_t)C * sizeof(float);
+    ZI_DISPATCH_DTYPE(proj_dt, TP, ZI_DISPATCH_DTYPE(dt, T, {
+        conv_qkv_kernel<TP, T><<<n, CQ_THREADS, lds, stream>>>(
+            (T*)q_out, ldq, (T*)kcache, (T*)vcache, (const TP*)proj, ld, bias, conv_w, state, state_stride, q_norm, k_norm,
+            eps, table, rot, tok_seq, entry_start, entry_slot, slots, cache_slots, nh, nkv, dim, vdim, D, taps, page_size);
+    }));
+    return zi_check_launch("conv_qkv");
+}
+
+// The convolution's new tail: the last taps - 1 rows of u = projection + bias of the sequence so far, from this
+// step's rows and, where the entry brought fewer, from the old tail.  A thread reads all it needs of the old tail
+// before it writes.
+template <typename TP>
+__global__ void __launch_bounds__(256)
+conv_tail_kernel(float* __restrict__ state, int64_t state_stride, const TP* __restrict__ proj, int64_t ld,
+                 const float* __restrict__ bias, const int32_t* __restrict__ entry_start,
+                 const int32_t* __restrict__ entry_len, const int32_t* __restrict__ entry_slot, int C, int taps) {
+    const int e = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int start = entry_start[e], len = entry_len[e];
+    float* tail = state + (int64_t)entry_slot[e] * state_stride;
+    const float bc = bias ? bias[c] : 0.f;
+    float keep[CQ_MAX_TAPS];
+#pragma unroll
+    for (int k = 0; k < CQ_MAX_TAPS; ++k) {
+        if (k >= taps - 1) break;
+        const int li = len - (taps - 1) + k;
+        keep[k] = li >= 0 ? zi_load(proj + (int64_t)(start + li) * ld + c) + bc : tail[(int64_t)(li + taps - 1) * C + c];
+    }
+#pragma unroll
+    for (int k = 0; k < CQ_MAX_TAPS; ++k) {
+        if (k >= taps - 1) break;
+        tail[(int64_t)k * C + c] = keep[k];
+    }
+}
+
+extern "C" int zi_conv_tail(float* state, int64_t state_stride, const void* proj, int proj_dt, int64_t ld,
+                            const float* bias, const int32_t* entry_start, const int32_t* entry_len,
+                            const int32_t* entry_slot, int entries, int channels, int taps, hipStream_t stream) {
+    ZI_REQUIRE(entries >= 0 && entries <= 65535 && channels > 0 && taps >= 1 && taps <= CQ_MAX_TAPS,
+               "conv_tail: bad sizes (at most %d taps)", CQ_MAX_TAPS);
+    ZI_REQUIRE(ld >= channels && state_stride >= (int64_t)(taps - 1) * channels, "conv_tail: a row is too short");
+    if (entries == 0 || taps == 1) return 0;
+    ZI_DISPATCH_DTYPE(proj_dt, TP, {
+        conv_tail_kernel<TP><<<dim3((channels + 255) / 256, entries), 256, 0, stream>>>(
+            state, state_stride, (const TP*)proj, ld, bias, entry_start, entry_len, entry_slot, channels, taps);
+    });
+    return zi_check_launch("conv_tail");
+}

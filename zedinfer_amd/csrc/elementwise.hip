@@ -236,3 +236,94 @@ extern "C" int zi_gated_act(void* out, int out_dt, int64_t ldo, const void* gate
     }));
     return zi_check_launch("gated_act");
 }
+
+// ---- activations of feed-forwards without the SiLU gate ------------------------------------------------------
+// relu(z)^2 of every element of a [n][inter] operand with dense rows, which may come as `splits` float32 partial
+// sums (split s at z + s * split_stride, added in rising order first).
+template <typename T, typename TO>
+__global__ void relu_squared_kernel(TO* __restrict__ out, int64_t ldo, const T* __restrict__ z, int64_t ldz, int splits,
+                                    int64_t split_stride, int n, int inter) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)n * inter) return;
+    const int64_t r = i / inter, c = i % inter;
+    float v = zi_load(z + r * ldz + c);
+    for (int s = 1; s < splits; ++s) v += zi_load(z + s * split_stride + r * ldz + c);
+    v = fmaxf(v, 0.f);
+    zi_store(out + r * ldo + c, v * v);
+}
+
+extern "C" int zi_relu_squared(void* out, int out_dt, int64_t ldo, const void* z, int dt, int64_t ldz, int splits,
+                               int64_t split_stride, int n, int inter, hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && inter > 0 && ldo >= inter && ldz >= inter && splits >= 1, "relu_squared: bad sizes");
+    if (n == 0) return 0;
+    const int64_t total = (int64_t)n * inter;
+    ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(out_dt, TO, {
+        relu_squared_kernel<T, TO><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(
+            (TO*)out, ldo, (const T*)z, ldz, splits, split_stride, n, inter);
+    }));
+    return zi_check_launch("relu_squared");
+}
+
+// The clamped gated activation: g = min(gate, limit), u = clamp(up, -limit, limit), out = g sigmoid(alpha g) (u + 1).
+// gate and up are [n][inter] with dense rows (column slices of one product are fine), possibly as `splits` float32
+// partial sums.
+template <typename T, typename TO>
+__global__ void clamped_glu_kernel(TO* __restrict__ out, int64_t ldo, const T* __restrict__ gate, const T* __restrict__ up,
+                                   int64_t ld_gate, int64_t ld_up, int splits, int64_t split_stride, int n, int inter,
+                                   float limit, float alpha) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= (int64_t)n * inter) return;
+    const int64_t r = i / inter, c = i % inter;
+    float g = zi_load(gate + r * ld_gate + c), u = zi_load(up + r * ld_up + c);
+    for (int s = 1; s < splits; ++s) {
+        g += zi_load(gate + s * split_stride + r * ld_gate + c);
+        u += zi_load(up + s * split_stride + r * ld_up + c);
+    }
+    g = fminf(g, limit);
+    u = fminf(fmaxf(u, -limit), limit);
+    zi_store(out + r * ldo + c, g / (1.f + expf(-alpha * g)) * (u + 1.f));
+}
+
+extern "C" int zi_clamped_glu(void* out, int out_dt, int64_t ldo, const void* gate, const void* up, int dt, int64_t ld_gate,
+                              int64_t ld_up, int splits, int64_t split_stride, int n, int inter, float limit, float alpha,
+                              hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && inter > 0 && ldo >= inter && ld_gate >= inter && ld_up >= inter && splits >= 1,
+               "clamped_glu: bad sizes");
+    ZI_REQUIRE(limit > 0.f, "clamped_glu: the limit must be positive, got %g", (double)limit);
+    if (n == 0) return 0;
+    const int64_t total = (int64_t)n * inter;
+    ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(out_dt, TO, {
+        clamped_glu_kernel<T, TO><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(
+            (TO*)out, ldo, (const T*)gate, (const T*)up, ld_gate, ld_up, splits, split_stride, n, inter, limit, alpha);
+    }));
+    return zi_check_launch("clamped_glu");
+}
+
+// x <- cap * tanh(x / cap), float32, in place (the soft cap of logits).
+__global__ void softcap_kernel(float* __restrict__ x, int64_t total, float cap) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) x[i] = cap * tanhf(x[i] / cap);
+}
+
+extern "C" int zi_softcap(float* x, int64_t total, float cap, hipStream_t stream) {
+    ZI_REQUIRE(total >= 0 && cap > 0.f, "softcap: bad sizes or cap %g", (double)cap);
+    if (total == 0) return 0;
+    softcap_kernel<<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(x, total, cap);
+    return zi_check_launch("softcap");
+}
+
+// out = x in another storage type (the rounded copy of float32 rows that a matrix product reads).
+template <typename T, typename TO>
+__global__ void convert_kernel(TO* __restrict__ out, const T* __restrict__ x, int64_t total) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < total) zi_store(out + i, zi_load(x + i));
+}
+
+extern "C" int zi_convert(void* out, int out_dt, const void* x, int dt, int64_t total, hipStream_t stream) {
+    ZI_REQUIRE(total >= 0, "convert: bad size");
+    if (total == 0) return 0;
+    ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(out_dt, TO, {
+        convert_kernel<T, TO><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>((TO*)out, (const T*)x, total);
+    }));
+    return zi_check_launch("convert");
+}

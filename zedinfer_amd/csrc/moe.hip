@@ -92,6 +92,72 @@ extern "C" int zi_moe_route(int32_t* idx, float* wt, const float* z, const float
     return zi_check_launch("moe_route");
 }
 
+// The other router: the `top` largest logits themselves are chosen (the lowest index among equals) and the weights
+// are the softmax over the chosen logits only.  z [n][E] float32; `bias` [E] (or null) is added to it first.
+template <int PER>
+__global__ void __launch_bounds__(256)
+moe_route_top_kernel(int32_t* __restrict__ idx, float* __restrict__ wt, const float* __restrict__ z,
+                     const float* __restrict__ bias, int n, int E, int top) {
+    const int lane = threadIdx.x % ZI_WAVE;
+    const int t = blockIdx.x * (blockDim.x / ZI_WAVE) + threadIdx.x / ZI_WAVE;
+    if (t >= n) return;
+    float choice[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+        const int e = lane + i * ZI_WAVE;
+        choice[i] = e < E ? z[(int64_t)t * E + e] + (bias ? bias[e] : 0.f) : -INFINITY;
+    }
+    float first = 0.f, sum = 0.f;
+    for (int k = 0; k < top; ++k) {
+        float best = -INFINITY;
+        int best_e = 0x7fffffff;
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int e = lane + i * ZI_WAVE;
+            if (e < E && (choice[i] > best || (choice[i] == best && e < best_e))) {
+                best = choice[i];
+                best_e = e;
+            }
+        }
+#pragma unroll
+        for (int o = ZI_WAVE / 2; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, ZI_WAVE);
+            const int oe = __shfl_xor(best_e, o, ZI_WAVE);
+            if (ob > best || (ob == best && oe < best_e)) {
+                best = ob;
+                best_e = oe;
+            }
+        }
+        if (k == 0) first = best;      // the largest of all: the softmax's maximum
+        const float p = expf(best - first);
+        sum += p;
+        if (lane == 0) {
+            idx[(int64_t)t * top + k] = best_e;
+            wt[(int64_t)t * top + k] = p;
+        }
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            if (lane + i * ZI_WAVE == best_e) choice[i] = -INFINITY;
+    }
+    if (lane == 0)
+        for (int k = 0; k < top; ++k) wt[(int64_t)t * top + k] /= sum;
+}
+
+extern "C" int zi_moe_route_top(int32_t* idx, float* wt, const float* z, const float* bias, int n, int experts, int top,
+                                hipStream_t stream) {
+    ZI_REQUIRE(n >= 0 && experts > 0 && experts <= MOE_MAX_EXPERTS && top > 0 && top <= experts,
+               "moe_route_top: bad sizes (experts %d, top %d; at most %d experts)", experts, top, MOE_MAX_EXPERTS);
+    if (n == 0) return 0;
+    const int blocks = (n + 3) / 4;
+#define ZI_MOE_ROUTE(PER) moe_route_top_kernel<PER><<<blocks, 256, 0, stream>>>(idx, wt, z, bias, n, experts, top)
+    if (experts <= ZI_WAVE) ZI_MOE_ROUTE(1);
+    else if (experts <= 2 * ZI_WAVE) ZI_MOE_ROUTE(2);
+    else if (experts <= 4 * ZI_WAVE) ZI_MOE_ROUTE(4);
+    else ZI_MOE_ROUTE(MOE_PER_LANE);
+#undef ZI_MOE_ROUTE
+    return zi_check_launch("moe_route_top");
+}
+
 // One workgroup sorts the M = n * top pairs by expert (a counting sort; within an expert the order is the order
 // of arrival, which no result depends on).  plan: [0] = number of row tiles, then [1 + 3 i ...] = (expert, first
 // row, rows) of tile i; order[place] = pair, place_of[pair] = place.

@@ -147,6 +147,49 @@ int zi_moe_linear(void* out, int out_dt, int64_t ldo, const void* x, int x_dt, i
 // moe.hip
 int zi_moe_combine(float* out, const float* y, const float* wt, const int32_t* place_of, int n, int top, int hidden,
     hipStream_t stream);
+// attention_generic.hip
+int zi_attention_generic_sink(void* out, const void* q, int dt, int n, int64_t ldq, int64_t ldo, const void* kcache,
+    const void* vcache, const int32_t* tok_index, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t*
+    block_tables, int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window, float scale, const
+    float* sinks, hipStream_t stream);
+// attention_decode.hip
+int zi_attention_decode_sink(void* out, const void* q, int dt, int n_idx, int64_t ldq, int64_t ldo, const void* kcache,
+    const void* vcache, const int32_t* tok_index, const int32_t* tok_seq, const int32_t* tok_pos, const int32_t*
+    block_tables, int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window, float scale, int
+    max_chunks, float* workspace, int64_t workspace_floats, const float* sinks, hipStream_t stream);
+// attention_prefill.hip
+int zi_attention_prefill_sink(void* out, const void* q, int dt, int num_tiles, int64_t ldq, int64_t ldo, const void*
+    kcache, const void* vcache, const int32_t* tile_entry, const int32_t* tile_off, const int32_t* entry_start, const
+    int32_t* entry_len, const int32_t* entry_past, const int32_t* block_tables, int max_pages, int num_pages, int nh,
+    int nkv, int d, int page_size, int window, float scale, int rows, int max_chunks, float* workspace, int64_t
+    workspace_floats, int tile, int alone, int chunk_keys, const float* sinks, hipStream_t stream);
+// layer_norm.hip
+int zi_layer_norm(void* out, int out_dt, int64_t ldo, float* resid, const void* x, int x_dt, int splits, int64_t
+    split_stride, int64_t ldx, const void* w, const void* b, int w_dt, int n, int hidden, float eps, hipStream_t
+    stream);
+// conv_qkv.hip
+int zi_conv_qkv(void* q_out, int dt, int64_t ldq, void* kcache, void* vcache, const void* proj, int proj_dt, int64_t ld,
+    const float* bias, const float* conv_w, const float* state, int64_t state_stride, const float* q_norm, const float*
+    k_norm, float eps, const float* table, int rot, int n, const int32_t* tok_seq, const int32_t* entry_start, const
+    int32_t* entry_slot, const int32_t* slots, int64_t cache_slots, int nh, int nkv, int dim, int vdim, int D, int taps,
+    int page_size, hipStream_t stream);
+// conv_qkv.hip
+int zi_conv_tail(float* state, int64_t state_stride, const void* proj, int proj_dt, int64_t ld, const float* bias, const
+    int32_t* entry_start, const int32_t* entry_len, const int32_t* entry_slot, int entries, int channels, int taps,
+    hipStream_t stream);
+// elementwise.hip
+int zi_relu_squared(void* out, int out_dt, int64_t ldo, const void* z, int dt, int64_t ldz, int splits, int64_t
+    split_stride, int n, int inter, hipStream_t stream);
+// elementwise.hip
+int zi_clamped_glu(void* out, int out_dt, int64_t ldo, const void* gate, const void* up, int dt, int64_t ld_gate, int64_t
+    ld_up, int splits, int64_t split_stride, int n, int inter, float limit, float alpha, hipStream_t stream);
+// elementwise.hip
+int zi_softcap(float* x, int64_t total, float cap, hipStream_t stream);
+// elementwise.hip
+int zi_convert(void* out, int out_dt, const void* x, int dt, int64_t total, hipStream_t stream);
+// moe.hip
+int zi_moe_route_top(int32_t* idx, float* wt, const float* z, const float* bias, int n, int experts, int top,
+    hipStream_t stream);
 // sampling.hip
 int zi_argmax(int32_t* out_idx, float* out_val, const void* logits, int dt, int rows, int vocab, int64_t ld, float*
     workspace, int64_t workspace_floats, hipStream_t stream);
@@ -196,5 +239,16 @@ int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int ro
     X(zi_moe_group) \
     X(zi_moe_linear) \
     X(zi_moe_combine) \
+    X(zi_attention_generic_sink) \
+    X(zi_attention_decode_sink) \
+    X(zi_attention_prefill_sink) \
+    X(zi_layer_norm) \
+    X(zi_conv_qkv) \
+    X(zi_conv_tail) \
+    X(zi_relu_squared) \
+    X(zi_clamped_glu) \
+    X(zi_softcap) \
+    X(zi_convert) \
+    X(zi_moe_route_top) \
     X(zi_argmax) \
     X(zi_sample)

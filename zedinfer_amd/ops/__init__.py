@@ -22,6 +22,8 @@ from .mixing import (delta_conv_state, delta_prepare, delta_rule, delta_state_fl
                      latent_attention, latent_attention_cores, latent_attention_cores_plan,
                      latent_attention_cores_supported, latent_attention_cores_workspace, latent_query, latent_store, latent_value, moe_combine, moe_group, moe_linear,
                      moe_max_tiles, moe_route, moe_tile_rows, rope_pairs)
+from .sublayers import (clamped_glu, conv_qkv, conv_state_floats, conv_tail, convert, layer_norm, moe_route_top,
+                        relu_squared, softcap)
 from ._lib import KernelLibraryError, library_path, load
 
 __all__ = [
@@ -39,5 +41,7 @@ __all__ = [
     "latent_attention", "latent_attention_cores", "latent_attention_cores_plan", "latent_attention_cores_supported",
     "latent_attention_cores_workspace", "latent_query", "latent_store", "latent_value", "moe_combine", "moe_group", "moe_linear",
     "moe_max_tiles", "moe_route", "moe_tile_rows", "rope_pairs",
+    "clamped_glu", "conv_qkv", "conv_state_floats", "conv_tail", "convert", "layer_norm", "moe_route_top", "relu_squared",
+    "softcap",
     "KernelLibraryError", "library_path", "load", "FEW_ROWS", "SUMS_MAX_ROWS",
 ]

@@ -85,6 +85,18 @@ _PROTOTYPES = {
     "zi_moe_group": [P, P, P, P, I, I, I, P],
     "zi_moe_linear": [P, I, L, P, I, L, P, I, P, P, I, I, I, I, I, I, P],
     "zi_moe_combine": [P, P, P, P, I, I, I, P],
+    "zi_attention_generic_sink": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, P, P],
+    "zi_attention_decode_sink": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P, L, P, P],
+    "zi_attention_prefill_sink": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, I, I, I,
+                                  P, P],
+    "zi_layer_norm": [P, I, L, P, P, I, I, L, L, P, P, I, I, I, F, P],
+    "zi_conv_qkv": [P, I, L, P, P, P, I, L, P, P, P, L, P, P, F, P, I, I, P, P, P, P, L, I, I, I, I, I, I, I, P],
+    "zi_conv_tail": [P, L, P, I, L, P, P, P, P, I, I, I, P],
+    "zi_relu_squared": [P, I, L, P, I, L, I, L, I, I, P],
+    "zi_clamped_glu": [P, I, L, P, P, I, L, L, I, L, I, I, F, F, P],
+    "zi_softcap": [P, L, F, P],
+    "zi_convert": [P, I, P, I, L, P],
+    "zi_moe_route_top": [P, P, P, P, I, I, I, P],
     "zi_tape_record": [P, c_char_p, P, I],
     "zi_tape_record_many": [P, c_char_p, P, P, I],
     "zi_tape_run": [P, P],

@@ -363,21 +363,33 @@ def _attention_args(what, q, kcache, vcache, tok_seq, tok_pos, block_tables, nh,
 
 def attention(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tok_seq: torch.Tensor,
               tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
-              window: int = 0, out: Optional[torch.Tensor] = None, tok_index: Optional[torch.Tensor] = None
-              ) -> torch.Tensor:
+              window: int = 0, out: Optional[torch.Tensor] = None, tok_index: Optional[torch.Tensor] = None,
+              sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """Causal grouped-query attention of q [n, nh*d] over the paged cache: the plain kernel, for
     every shape and both storage types.
 
     Token i belongs to row ``tok_seq[i]`` of ``block_tables`` [seqs, max_pages] and sits at
     absolute position ``tok_pos[i]``; it sees the cached keys at positions
     [max(0, pos - window + 1), pos] (window 0: all of them).  With ``tok_index`` only the listed
-    tokens are computed (the other rows of ``out`` are left alone).  Returns [n, nh*d]."""
+    tokens are computed (the other rows of ``out`` are left alone).  ``sinks`` (float32 [nh]): the softmax of
+    head h also counts exp(sinks[h]) in its denominator, a term with no key and no value.  Returns [n, nh*d]."""
     out, n, count, ldq, ldo, pages, ps = _attention_args("attention", q, kcache, vcache, tok_seq, tok_pos,
                                                          block_tables, nh, nkv, d, tok_index, out)
-    _lib.call("zi_attention_generic", _p(out), _p(q), _code(q, "attention"), count, ldq, ldo, _p(kcache), _p(vcache),
-              _p(tok_index), _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages, nh, nkv, d,
-              ps, int(window), float(scale), _stream())
+    args = (_p(out), _p(q), _code(q, "attention"), count, ldq, ldo, _p(kcache), _p(vcache),
+            _p(tok_index), _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages, nh, nkv, d,
+            ps, int(window), float(scale))
+    if sinks is not None:
+        _lib.call("zi_attention_generic_sink", *args, _p(_sinks(sinks, nh, q, "attention")), _stream())
+    else:
+        _lib.call("zi_attention_generic", *args, _stream())
     return out
+
+
+def _sinks(sinks: torch.Tensor, nh: int, q: torch.Tensor, what: str) -> torch.Tensor:
+    if sinks.dtype != torch.float32 or sinks.dim() != 1 or sinks.numel() != nh or not sinks.is_contiguous() \
+            or sinks.device != q.device:
+        raise ValueError(f"{what}: sinks must be a contiguous float32 [{nh}] tensor on {q.device}")
+    return sinks
 
 
 
@@ -402,8 +414,8 @@ def attention_decode_workspace(tokens: int, nh: int, d: int) -> int:
 def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, tok_seq: torch.Tensor,
                      tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                      max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None,
-                     tok_index: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None
-                     ) -> torch.Tensor:
+                     tok_index: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
+                     sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The same attention for single query tokens, split over the keys, on the matrix cores
     (bfloat16, head_dim a multiple of 16 up to 128, group size <= 16, page size a multiple of 8).
     ``max_keys`` is an upper bound of the keys any listed token sees (its position + 1), known on
@@ -419,10 +431,14 @@ def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
             workspace = torch.empty((need,), dtype=torch.float32, device=q.device)
         if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
             raise ValueError(f"attention_decode: workspace must be a contiguous float32 buffer of {need} entries")
-    _lib.call("zi_attention_decode", _p(out), _p(q), _code(q, "attention_decode"), count, ldq, ldo, _p(kcache),
-              _p(vcache), _p(tok_index), _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages,
-              nh, nkv, d, ps, int(window), float(scale), max_chunks, _p(workspace),
-              workspace.numel() if workspace is not None else 0, _stream())
+    args = (_p(out), _p(q), _code(q, "attention_decode"), count, ldq, ldo, _p(kcache),
+            _p(vcache), _p(tok_index), _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages,
+            nh, nkv, d, ps, int(window), float(scale), max_chunks, _p(workspace),
+            workspace.numel() if workspace is not None else 0)
+    if sinks is not None:      # (float32 [nh]: exp(sinks[h]) counts once in head h's denominator)
+        _lib.call("zi_attention_decode_sink", *args, _p(_sinks(sinks, nh, q, "attention_decode")), _stream())
+    else:
+        _lib.call("zi_attention_decode", *args, _stream())
     return out
 
 
@@ -710,7 +726,8 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
                       tile_off: torch.Tensor, entry_start: torch.Tensor, entry_len: torch.Tensor,
                       entry_past: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                       window: int = 0, out: Optional[torch.Tensor] = None, max_keys: int = 0,
-                      workspace: Optional[torch.Tensor] = None, tile: int = 0, alone: bool = False) -> torch.Tensor:
+                      workspace: Optional[torch.Tensor] = None, tile: int = 0, alone: bool = False,
+                      sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The same attention for portions of prompts, on the matrix cores (bfloat16, head_dim a multiple
     of 16 up to 128, page size a power of two from 8).
 
@@ -760,11 +777,15 @@ def attention_prefill(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tenso
             workspace = torch.empty((need,), dtype=torch.float32, device=q.device)
         if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
             raise ValueError(f"attention_prefill: workspace must be a contiguous float32 buffer of {need} entries")
-    _lib.call("zi_attention_prefill", _p(out), _p(q), _code(q, "attention_prefill"), num_tiles, ldq, ldo, _p(kcache),
-              _p(vcache), _p(tile_entry), _p(tile_off), _p(entry_start), _p(entry_len), _p(entry_past),
-              _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale), n,
-              max_chunks, _p(workspace) if need else _p(None), workspace.numel() if need else 0, int(tile), int(bool(alone)),
-              chunk_keys, _stream())
+    args = (_p(out), _p(q), _code(q, "attention_prefill"), num_tiles, ldq, ldo, _p(kcache),
+            _p(vcache), _p(tile_entry), _p(tile_off), _p(entry_start), _p(entry_len), _p(entry_past),
+            _p(block_tables), block_tables.shape[1], pages, nh, nkv, d, ps, int(window), float(scale), n,
+            max_chunks, _p(workspace) if need else _p(None), workspace.numel() if need else 0, int(tile), int(bool(alone)),
+            chunk_keys)
+    if sinks is not None:      # (float32 [nh]: exp(sinks[h]) counts once in head h's denominator)
+        _lib.call("zi_attention_prefill_sink", *args, _p(_sinks(sinks, nh, q, "attention_prefill")), _stream())
+    else:
+        _lib.call("zi_attention_prefill", *args, _stream())
     return out
 
 

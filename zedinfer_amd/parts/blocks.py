@@ -75,3 +75,50 @@ class ParallelBlock(Block):
         if self.has_ff:
             self._term(terms[1], self.feed_forward, x)
         return terms
+
+
+@register_block("output_norm")
+class OutputNormBlock(Block):
+    """h += norm_mixer(mixer(h)); h += norm_ff(feed_forward(h)): the sublayers read the residual stream itself (its
+    rounding to the activation type, where that is not float32) and the norm sits on each sublayer's output.  The
+    norms must offer ``add_normed`` (the layer norm does).  Nothing is left pending: the stream is whole when the
+    block returns.  The rounded copy of the stream that the last norm left is handed to the next block of the kind
+    through ``batch.shared``, which holds for one run of the model.  The feed-forward may be the kind "none"."""
+
+    graph_safe = True
+    tape_safe = True
+
+    norm_names = ("mixer_out", "ff_out")
+    SHARED = "output_norm_block.resid_copy"
+
+    def __init__(self, norms, mixer, feed_forward, rt: Runtime):
+        self.norm_mixer = norms["mixer_out"]
+        self.norm_ff = norms["ff_out"]
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.has_ff = getattr(feed_forward, "kind", "") != "none"
+        self.rt = rt
+
+    def _copy_of(self, resid: torch.Tensor, batch) -> torch.Tensor:
+        if self.rt.dtype == torch.float32:
+            return resid
+        shared = getattr(batch, "shared", None)
+        x = shared.get(self.SHARED) if shared is not None else None
+        if x is None:
+            x = ops.convert(resid, self.rt.buffer("resid_copy", tuple(resid.shape), self.rt.dtype))
+        return x
+
+    def forward(self, resid: torch.Tensor, delta: Optional[torch.Tensor], batch, memory: LayerMemory):
+        if delta is not None:       # a block of another kind before this one left an addition pending
+            for term in (delta if delta.dim() == 3 else (delta,)):
+                ops.add(resid, term, out=resid)
+        x = self._copy_of(resid, batch)
+        a = self.mixer.forward(x, batch, memory)
+        x = self.norm_mixer.add_normed(resid, a)
+        if self.has_ff:
+            f = self.feed_forward.forward(x if x is not None else resid)
+            x = self.norm_ff.add_normed(resid, f)
+        shared = getattr(batch, "shared", None)
+        if shared is not None:
+            shared[self.SHARED] = x
+        return None

@@ -47,7 +47,8 @@ class LinearHead(Part):
     """logits = x . W^T in float32, no bias (reference: transformer_forward.cpp:155-156).  With
     ``tied_to`` in the spec's weights the checkpoint may leave the tensor out and the embedding
     table stands in (reference: src/frontend/models/base.cpp:410-416).
-    params: vocab_size, hidden_size, tied_to (tensor name or None)."""
+    With ``softcap`` c the logits are then bounded smoothly: c * tanh(logits / c).
+    params: vocab_size, hidden_size, tied_to (tensor name or None), softcap (None)."""
 
     graph_safe = True
     tape_safe = True
@@ -61,7 +62,12 @@ class LinearHead(Part):
         super().__init__(spec, weights, rt)
         self.weight = weights["weight"]
         self.vocab = self.weight.shape[0]
+        cap = spec.params.get("softcap")
+        self.softcap = float(cap) if cap else None
 
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         out = self.rt.buffer("logits", (x.shape[0], self.vocab), torch.float32)
-        return ops.linear(x, self.weight, out=out)
+        ops.linear(x, self.weight, out=out)
+        if self.softcap is not None:
+            ops.softcap(out, self.softcap)
+        return out

@@ -286,3 +286,157 @@ class RoutedExperts(FeedForward):
         if out is None:
             out = rt.buffer("moe_out", (n, self.hidden), torch.float32)
         return ops.moe_combine(y, wt, place_of, out)
+
+
+def _float_result(rt: Runtime, name: str, x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """x . weight^T with float32 results for a norm to read: partial sums [S, n, N] for few rows, else [n, N]."""
+    n, N = x.shape[0], weight.shape[0]
+    if ops.linear_sums_supported(x, weight):
+        S = ops.linear_splits(n, N, x.shape[1])
+        return ops.linear_sums(x, weight, out=rt.buffer(name + "_sums", (S, n, N), torch.float32))
+    return ops.linear(x, weight, out=rt.buffer(name, (n, N), torch.float32))
+
+
+@register_feed_forward("relu2_mlp")
+class ReluSquaredMLP(FeedForward):
+    """down(relu(up(x))^2), no gate, no biases.  The result is float32 (partial sums for few rows): a norm reads it.
+    params: hidden_size, intermediate_size."""
+
+    graph_safe = True
+    tape_safe = True
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        H, I = int(spec.params["hidden_size"]), int(spec.params["intermediate_size"])
+        return {"up": WeightSpec((I, H)), "down": WeightSpec((H, I))}
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        self.hidden = int(spec.params["hidden_size"])
+        self.inter = int(spec.params["intermediate_size"])
+        self.up, self.down = weights["up"], weights["down"]
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        return ProductRows.step_rows(rows, kind)
+
+    def tune(self, num_tokens: int) -> None:
+        n = int(num_tokens)
+        self.rt.tune_linear(self.rt.buffer("resid_copy", (n, self.hidden)), self.up)
+        self.rt.tune_linear(self.rt.buffer("ffn_act", (n, self.inter)), self.down, out_dtype=torch.float32)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        n, I, rt = x.shape[0], self.inter, self.rt
+        act = rt.buffer("ffn_act", (n, I))
+        if ops.linear_sums_supported(x, self.up):
+            S = ops.linear_splits(n, I, self.hidden)
+            z = ops.linear_sums(x, self.up, out=rt.buffer("ffn_up_sums", (S, n, I), torch.float32))
+        else:
+            z = ops.linear(x, self.up, out=rt.buffer("ffn_up", (n, I)))
+        ops.relu_squared(z, out=act)
+        return _float_result(rt, "ffn_out_f32", act, self.down)
+
+
+class _ClampedGated:
+    """One feed-forward of the clamped gated form, down(g sigmoid(1.702 g) (u + 1)) with g = min(gate x, limit) and
+    u = clamp(up x, -limit, limit): gate and up stacked into one product (the up rows begin at a multiple of 8)."""
+
+    def __init__(self, gate: torch.Tensor, up: torch.Tensor, down: torch.Tensor, limit: float):
+        self.inter, self.hidden = int(gate.shape[0]), int(gate.shape[1])
+        self.up_at = -(-self.inter // 8) * 8
+        stacked = torch.zeros((self.up_at + self.inter, self.hidden), dtype=gate.dtype, device=gate.device)
+        stacked[:self.inter] = gate
+        stacked[self.up_at:] = up.to(gate.dtype)
+        self.gate_up, self.down, self.limit = stacked, down, float(limit)
+
+    def forward(self, rt: Runtime, x: torch.Tensor, name: str) -> torch.Tensor:
+        n, I = x.shape[0], self.inter
+        gu = ops.linear(x, self.gate_up, out=rt.buffer(name + "_gate_up", (n, self.up_at + I), torch.float32))
+        act = rt.buffer(name + "_act", (n, I))
+        ops.clamped_glu(gu[:, :I], gu[:, self.up_at:], self.limit, out=act)
+        return act
+
+
+@register_feed_forward("clamped_experts")
+class ClampedExperts(FeedForward):
+    """A mixture of small clamped gated feed-forwards (see ``_ClampedGated``; no biases) of which every token uses
+    ``top``, plus, optionally, a shared one that every token uses.
+
+    Router: z = W_router x + b in float32; the ``top`` experts with the largest z are chosen (the lowest index among
+    equals) and weighted by the softmax over the chosen logits only.  The result is the weighted sum of the chosen
+    experts' outputs plus the shared expert's, handed on as a stack of float32 terms [routed, shared].
+
+    Routing, grouping and the experts' products run on the device as for ``routed_experts`` (``csrc/moe.hip``): the
+    launches of a step do not depend on what the tokens choose.  The experts' matrices are stacked [E, 2 ff, H] (gate
+    rows, then up rows) and [E, H, ff] at load.
+    params: hidden_size, experts, top, ff, limit, shared_ff (0: none), shared_limit."""
+
+    graph_safe = True
+    tape_safe = True
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        p = spec.params
+        H, E, ff, sff = int(p["hidden_size"]), int(p["experts"]), int(p["ff"]), int(p.get("shared_ff", 0) or 0)
+        w = {"router": WeightSpec((E, H)), "router_bias": WeightSpec((E,), init="zeros")}
+        for e in range(E):
+            w[f"gate_{e}"] = WeightSpec((ff, H))
+            w[f"up_{e}"] = WeightSpec((ff, H))
+            w[f"down_{e}"] = WeightSpec((H, ff))
+        if sff:
+            w.update({"shared_gate": WeightSpec((sff, H)), "shared_up": WeightSpec((sff, H)),
+                      "shared_down": WeightSpec((H, sff))})
+        return w
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        p = spec.params
+        self.hidden, self.experts, self.top, self.ff = int(p["hidden_size"]), int(p["experts"]), int(p["top"]), int(p["ff"])
+        self.limit = float(p["limit"])
+        if not (0 < self.top <= self.experts):
+            raise ValueError(f"clamped_experts: top {self.top} of {self.experts} experts")
+        self.router = weights["router"]
+        self.router_bias = weights["router_bias"].float().contiguous()
+        E = self.experts
+        self.gate_up = torch.stack([torch.cat([weights[f"gate_{e}"], weights[f"up_{e}"].to(weights[f"gate_{e}"].dtype)])
+                                    for e in range(E)]).contiguous()
+        self.down = torch.stack([weights[f"down_{e}"] for e in range(E)]).contiguous()
+        self.shared = None
+        if int(p.get("shared_ff", 0) or 0):
+            self.shared = _ClampedGated(weights["shared_gate"], weights["shared_up"], weights["shared_down"],
+                                        float(p["shared_limit"]))
+
+    def step_rows(self, rows: int, kind: str) -> int:
+        return ProductRows.step_rows(rows, kind)
+
+    def tune(self, num_tokens: int) -> None:
+        n = int(num_tokens)
+        if self.shared is not None:
+            self.rt.tune_linear(self.rt.buffer("resid_copy", (n, self.hidden)), self.shared.gate_up, out_dtype=torch.float32)
+            self.rt.tune_linear(self.rt.buffer("moe_shared_act", (n, self.shared.inter)), self.shared.down,
+                                out_dtype=torch.float32)
+
+    def forward(self, x: torch.Tensor) -> torch.Tensor:
+        n, E, top, ff, rt = x.shape[0], self.experts, self.top, self.ff, self.rt
+        pairs = n * top
+        terms = rt.buffer("moe_terms", (2 if self.shared is not None else 1, n, self.hidden), torch.float32)
+        z = ops.linear(x, self.router, out=rt.buffer("moe_logits", (n, E), torch.float32))
+        idx = rt.buffer("moe_choice", (n, top), torch.int32)
+        wt = rt.buffer("moe_weight", (n, top), torch.float32)
+        ops.moe_route_top(z, self.router_bias, top, idx, wt)
+        rows = ops.moe_tile_rows(x.dtype, self.gate_up.dtype, (self.hidden, ff), pairs, E)
+        tiles = ops.moe_max_tiles(pairs, E, rows)
+        plan = rt.buffer("moe_plan", (1 + 3 * tiles,), torch.int32)
+        order = rt.buffer("moe_order", (pairs,), torch.int32)
+        place_of = rt.buffer("moe_place", (pairs,), torch.int32)
+        ops.moe_group(idx, E, rows, plan, order, place_of)
+        gu = rt.buffer("moe_gate_up", (pairs, 2 * ff), torch.float32)
+        ops.moe_linear(x, self.gate_up, plan, rows, tiles, out=gu, source=order, source_div=top)
+        act = rt.buffer("moe_act", (pairs, ff))
+        ops.clamped_glu(gu[:, :ff], gu[:, ff:], self.limit, out=act)
+        y = rt.buffer("moe_out_rows", (pairs, self.hidden), torch.float32)
+        ops.moe_linear(act, self.down, plan, rows, tiles, out=y)
+        ops.moe_combine(y, wt, place_of, terms[0])
+        if self.shared is not None:
+            act_s = self.shared.forward(rt, x, "moe_shared")
+            ops.linear(act_s, self.shared.down, out=terms[1])
+        return terms

@@ -10,8 +10,8 @@ import torch
 from .. import ops
 from ..config.forward_config import PartSpec
 from ..weights.loader import WeightSpec
-from .base import (PAGE, HostBatch, KVCacheRequest, LayerMemory, Mixer, PageTensor, POSITION_ENCODINGS, Runtime, StepPlan,
-                   StepPlanner, register_mixer)
+from .base import (PAGE, HostBatch, KVCacheRequest, LayerMemory, Mixer, PageTensor, POSITION_ENCODINGS, Runtime, StateRequest,
+                   StepPlan, StepPlanner, register_mixer)
 from .rows import ProductRows
 from .feed_forward import stack_rows
 
@@ -159,6 +159,8 @@ class Attention(Mixer):
     # the plain product does (measured: 6.9 against 4.4 + 3.7 us with 4.7 MB of weight, 31.7 against
     # about 16 us with 52 MB), so it is taken for small output weights only.
     PROJECT_FROM_CHUNKS_MAX_BYTES = 8 << 20
+    # float32 [heads] in mixers whose softmax counts exp(sink) of a learned number per head in its denominator
+    sinks: Optional[torch.Tensor] = None
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
@@ -224,11 +226,12 @@ class Attention(Mixer):
                 ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n_short, self.nh, self.d),),
                                     torch.float32)
                 ops.attention_decode(q, *args, plan.sizes["max_short_keys"], self.window, out=att,
-                                     tok_index=plan.dev["short_idx"] if n_short < N else None, workspace=ws)
+                                     tok_index=plan.dev["short_idx"] if n_short < N else None, workspace=ws,
+                                     sinks=self.sinks)
             else:
                 n_long = -1      # everything through the plain kernel
         if n_long < 0:
-            ops.attention(q, *args, self.window, out=att)
+            ops.attention(q, *args, self.window, out=att, sinks=self.sinks)
         elif n_long > 0:
             if ops.attention_prefill_supported(q.dtype, self.nh, self.nkv, self.d, kc.shape[2]):
                 max_keys = plan.sizes["max_long_keys"]
@@ -238,9 +241,10 @@ class Attention(Mixer):
                 ops.attention_prefill(q, kc, vc, plan.dev["tile_entry"], plan.dev["tile_off"],
                                       batch.entry_start, batch.entry_len, batch.entry_past, view.block_tables, self.nh,
                                       self.nkv, self.d, self.scale, self.window, out=att, max_keys=max_keys,
-                                      workspace=ws, tile=plan.sizes["tile"], alone=plan.sizes["alone"])
+                                      workspace=ws, tile=plan.sizes["tile"], alone=plan.sizes["alone"], sinks=self.sinks)
             else:
-                ops.attention(q, *args, self.window, out=att, tok_index=plan.dev["long_idx"] if n_long < N else None)
+                ops.attention(q, *args, self.window, out=att, tok_index=plan.dev["long_idx"] if n_long < N else None,
+                              sinks=self.sinks)
 
     def planner(self) -> StepPlanner:
         return attention_planner(self.wide_tile, self.nh)
@@ -381,4 +385,110 @@ class Attention(Mixer):
                                                 out=out)
         att = self.rt.buffer("attn_out", (n, self.qd))
         ops.attention_decode_fused(*args, out=att, workspace=ws, write_kv=memory.writes)
+        return self.project(att, n)
+
+
+@register_mixer("conv_attention")
+class ConvAttention(Attention):
+    """Causal grouped-query attention whose projections pass a short convolution, with a sink in the softmax.
+
+    q, k, v = W x + b; each channel then passes a causal convolution over time (``conv`` taps, no bias, zeros before
+    the sequence's start); q and k are RMS-normed over the WHOLE projection (all heads at once, gains of that size);
+    the first ``rotary_dim`` dims of every head of q and k turn (the position encoding must hand over a table of
+    split-half angles, or do nothing); scores are (q . k) * ``scale`` over all earlier positions (or a window); the
+    softmax's denominator also holds exp(sink_h), a learned number per head without key or value; W_o on the
+    concatenated heads.  Keys have ``head_dim`` values a head, values ``value_dim``.
+
+    The cache holds heads of one size, the larger of the two rounded up to what the matrix-core kernels take (a
+    multiple of 16 up to 128 in bfloat16); the shorter kind is followed by zeros, which change no score and no
+    output, and W_o gets zero columns where the padding stands.  A request's state is the last conv - 1 rows that
+    entered the convolution (float32, the biases in them).  Everything between the projection and the attention
+    kernels is one launch in float32 arithmetic (``csrc/conv_qkv.hip``); the projections leave float32 results.
+    Steps of such a model are never padded: a padding token would move the convolution's tail.
+
+    params: hidden_size, num_heads, num_kv_heads, head_dim, value_dim, conv, scale, window (0), eps, position."""
+
+    padding_safe = False
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        p = spec.params
+        H, nh, nkv, d, dv, taps = (int(p[k]) for k in ("hidden_size", "num_heads", "num_kv_heads", "head_dim",
+                                                      "value_dim", "conv"))
+        return {"q": WeightSpec((nh * d, H)), "k": WeightSpec((nkv * d, H)), "v": WeightSpec((nkv * dv, H)),
+                "q_bias": WeightSpec((nh * d,)), "k_bias": WeightSpec((nkv * d,)), "v_bias": WeightSpec((nkv * dv,)),
+                "q_conv": WeightSpec((nh * d, taps)), "k_conv": WeightSpec((nkv * d, taps)),
+                "v_conv": WeightSpec((nkv * dv, taps)),
+                "q_norm": WeightSpec((nh * d,), init="ones"), "k_norm": WeightSpec((nkv * d,), init="ones"),
+                "sink": WeightSpec((nh,), init="zeros"), "o": WeightSpec((H, nh * dv))}
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        Mixer.__init__(self, spec, weights, rt)
+        p = spec.params
+        self.hidden = int(p["hidden_size"])
+        self.nh, self.nkv = int(p["num_heads"]), int(p["num_kv_heads"])
+        self.dim, self.vdim, self.taps = int(p["head_dim"]), int(p["value_dim"]), int(p["conv"])
+        if self.nh % self.nkv:
+            raise ValueError(f"conv_attention: {self.nh} heads are not a multiple of {self.nkv} key/value heads")
+        if not (1 <= self.taps <= ops.sublayers.CONV_MAX_TAPS):
+            raise ValueError(f"conv_attention: conv must lie in 1..{ops.sublayers.CONV_MAX_TAPS}")
+        self.window = int(p.get("window", 0) or 0)
+        self.scale = float(p["scale"])
+        self.eps = float(p["eps"])
+        # the one head size of the cache and of the attention kernels
+        big = max(self.dim, self.vdim)
+        self.d = -(-big // 16) * 16 if (rt.dtype == torch.bfloat16 and big <= 128) else big
+        self.qd, self.kvd = self.nh * self.d, self.nkv * self.d
+        self.channels = self.nh * self.dim + self.nkv * self.dim + self.nkv * self.vdim
+        if self.channels > ops.sublayers.CONV_MAX_CHANNELS:
+            raise ValueError(f"conv_attention: {self.channels} channels are more than {ops.sublayers.CONV_MAX_CHANNELS}")
+        pos_spec: PartSpec = p["position"]
+        self.position = POSITION_ENCODINGS.get(pos_spec.kind)(pos_spec, {}, rt)
+        mats = [weights["q"], weights["k"], weights["v"]]
+        self.qkv = torch.cat([m.to(mats[0].dtype) for m in mats], dim=0).contiguous()
+        self.bias = torch.cat([weights[k].float() for k in ("q_bias", "k_bias", "v_bias")]).contiguous()
+        self.conv_w = torch.cat([weights[k].float() for k in ("q_conv", "k_conv", "v_conv")]).contiguous()
+        self.q_norm, self.k_norm = weights["q_norm"].float().contiguous(), weights["k_norm"].float().contiguous()
+        self.sinks = weights["sink"].float().contiguous()
+        o = weights["o"]
+        if self.d != self.vdim:        # zero columns where the heads' padding stands
+            wide = torch.zeros((self.hidden, self.nh, self.d), dtype=o.dtype, device=o.device)
+            wide[:, :, :self.vdim] = o.view(self.hidden, self.nh, self.vdim)
+            o = wide.view(self.hidden, self.qd).contiguous()
+        self.o = o
+        self.qk_norm = False
+        self.wide_tile = ops.attention_prefill_tile(rt.dtype, self.d) if rt.device.type == "cuda" else LONG_TILE
+        self.plan_key = attention_planner(self.wide_tile, self.nh).key
+
+    def state_request(self) -> Optional[StateRequest]:
+        return StateRequest((ops.conv_state_floats(self.channels, self.taps),), torch.float32)
+
+    def tune(self, num_tokens: int) -> None:
+        n = int(num_tokens)
+        self.rt.tune_linear(self.rt.buffer("resid_copy", (n, self.hidden)), self.qkv, out_dtype=torch.float32)
+        self.rt.tune_linear(self.rt.buffer("attn_out", (n, self.qd)), self.o, out_dtype=torch.float32)
+
+    def project(self, att: torch.Tensor, n: int) -> torch.Tensor:
+        """W_o with float32 results (a norm reads them): partial sums for few rows, else one product."""
+        if ops.linear_sums_supported(att, self.o):
+            S = ops.linear_splits(n, self.hidden, self.qd)
+            return ops.linear_sums(att, self.o, out=self.rt.buffer("attn_proj_sums", (S, n, self.hidden), torch.float32))
+        return ops.linear(att, self.o, out=self.rt.buffer("attn_proj_f32", (n, self.hidden), torch.float32))
+
+    def forward(self, x: torch.Tensor, batch, memory: LayerMemory) -> torch.Tensor:
+        n, rt = x.shape[0], self.rt
+        view = batch.groups[memory.group]
+        table = self.position.step_table(batch)
+        if table is None:
+            raise ValueError("conv_attention: the position encoding must hand over a table of split-half angles")
+        proj = ops.linear(x, self.qkv, out=rt.buffer("conv_attn_proj", (n, self.channels), torch.float32))
+        q = rt.buffer("attn_q", (n, self.qd))
+        writes = memory.writes
+        ops.conv_qkv(proj, self.bias, self.conv_w, memory.state, self.q_norm, self.k_norm, self.eps,
+                     None if isinstance(table, str) else table, batch.tok_seq, batch.entry_start, batch.entry_slot,
+                     view.slots if writes else None, memory.tensors["k"] if writes else None,
+                     memory.tensors["v"] if writes else None, self.nh, self.nkv, self.dim, self.vdim, self.d, self.taps, q)
+        ops.conv_tail(memory.state, proj, self.bias, batch.entry_start, batch.entry_len, batch.entry_slot, self.taps)
+        att = rt.buffer("attn_out", (n, self.qd))
+        self.attend(q, att, batch, view, memory)
         return self.project(att, n)

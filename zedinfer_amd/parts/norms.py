@@ -40,3 +40,45 @@ class RMSNorm(Norm):
     def add_forward(self, resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
         out = self.rt.buffer("norm_out", (resid.shape[0], self.dim), self.rt.dtype)
         return ops.add_rms_norm(resid, delta, self.weight, self.eps, out=out, add_one=self.add_one)
+
+
+@register_norm("layernorm")
+class LayerNorm(Norm):
+    """y = (x - mean) / sqrt(var + eps) * w + b, var the mean of the squared deviations, all in float32.
+    params: dim, eps.  Beside the norm's two usual forms it has a third, ``add_normed(resid, y)``: the norm sits on a
+    sublayer's OUTPUT, resid += norm(y), and the new residual rows come back in the activation type (what the next
+    sublayer's products read)."""
+
+    graph_safe = True
+    tape_safe = True
+
+    @staticmethod
+    def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
+        dim = int(spec.params["dim"])
+        return {"weight": WeightSpec((dim,), init="ones"), "bias": WeightSpec((dim,), init="zeros")}
+
+    def __init__(self, spec: PartSpec, weights: Dict[str, torch.Tensor], rt: Runtime):
+        super().__init__(spec, weights, rt)
+        self.dim = int(spec.params["dim"])
+        self.eps = float(spec.params["eps"])
+        self.weight = weights["weight"]
+        self.bias = weights["bias"].to(self.weight.dtype)
+
+    def forward(self, x: torch.Tensor, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+        out = self.rt.buffer("norm_out", (x.shape[-2], self.dim), out_dtype or self.rt.dtype)
+        return ops.layer_norm(x, self.weight, self.bias, self.eps, out=out)
+
+    def add_forward(self, resid: torch.Tensor, delta: torch.Tensor) -> torch.Tensor:
+        for term in (delta if delta.dim() == 3 else (delta,)):
+            ops.add(resid, term, out=resid)
+        return self.forward(resid)
+
+    def add_normed(self, resid: torch.Tensor, y: torch.Tensor, want_copy: bool = True) -> Optional[torch.Tensor]:
+        """resid (float32, in place) += norm(y); y is [n, dim] or a stack [S, n, dim] of float32 terms that are added
+        first.  Returns the new residual rows in the activation type, or nothing when that type is float32 (the
+        stream itself serves) or no copy is wanted."""
+        out = None
+        if want_copy and self.rt.dtype != torch.float32:
+            out = self.rt.buffer("resid_copy", (resid.shape[0], self.dim), self.rt.dtype)
+        ops.layer_norm(y, self.weight, self.bias, self.eps, out=out, resid=resid)
+        return out

@@ -11,12 +11,33 @@ from ..config.forward_config import PartSpec
 from .base import PositionEncoding, Runtime, register_position_encoding
 
 
+def stretched_frequencies(rotary_dim: int, theta: float, scaling) -> np.ndarray:
+    """f_i = theta^(-2i / rotary_dim) in double precision, with the frequencies of long wavelengths divided:
+    with wavelength l = 2 pi / f, f stays where l < original / high, becomes f / factor where l > original / low,
+    and between the two is (1 - s) f / factor + s f with s = (original / l - low) / (high - low).  Rounded to
+    float32 once, at the end."""
+    missing = [k for k in ("factor", "low", "high", "original") if k not in scaling]
+    if missing:
+        raise ValueError("rope scaling lacks " + ", ".join(missing))
+    factor, low, high, orig = (float(scaling[k]) for k in ("factor", "low", "high", "original"))
+    if not (factor > 0 and high > low and orig > 0):
+        raise ValueError("rope scaling: factor and original must be positive, high above low")
+    i = np.arange(rotary_dim // 2, dtype=np.float64)
+    f = np.power(float(theta), -2.0 * i / rotary_dim)
+    wavelength = 2.0 * np.pi / f
+    s = (orig / wavelength - low) / (high - low)
+    mixed = (1.0 - s) * f / factor + s * f
+    out = np.where(wavelength < orig / high, f, np.where(wavelength > orig / low, f / factor, mixed))
+    return out.astype(np.float32)
+
+
 @register_position_encoding("rope_neox")
 class RopeNeox(PositionEncoding):
     """Split-half rotary encoding: pairs (k, k + R/2) of the first R = ``rotary_dim`` dims of
     each head turn by pos * theta^(-2k/R) (reference: src/backend/ops/rope/cpu/rope_cpu.cpp:12-66;
     the reference rotates the whole head, no scaling: rope_nvidia.cu:50).
-    params: head_dim, theta, rotary_dim (default head_dim)."""
+    params: head_dim, theta, rotary_dim (default head_dim), scaling (None, or a dict factor / low / high /
+    original: long wavelengths are stretched, ``stretched_frequencies``)."""
 
     graph_safe = True
     tape_safe = True
@@ -28,13 +49,18 @@ class RopeNeox(PositionEncoding):
         self.theta = float(spec.params["theta"])
         if self.rotary_dim % 2 or not (0 < self.rotary_dim <= self.head_dim):
             raise ValueError(f"rope_neox: rotary_dim {self.rotary_dim} must be even and within head_dim {self.head_dim}")
-        self.inv_freq = ops.rope_inv_freq(self.rotary_dim, self.theta, rt.device)
+        scaling = spec.params.get("scaling")
+        self.scaling = tuple(sorted((str(k), float(v)) for k, v in scaling.items())) if scaling else None
+        if self.scaling is None:
+            self.inv_freq = ops.rope_inv_freq(self.rotary_dim, self.theta, rt.device)
+        else:
+            self.inv_freq = torch.from_numpy(stretched_frequencies(self.rotary_dim, self.theta, dict(self.scaling))).to(rt.device)
 
     def step_table(self, batch):
-        key = ("rope_neox", self.rotary_dim, self.theta)
+        key = ("rope_neox", self.rotary_dim, self.theta, self.scaling)
         table = batch.shared.get(key)
         if table is None:
-            out = self.rt.buffer(f"rope_table_{self.rotary_dim}_{self.theta!r}",
+            out = self.rt.buffer(f"rope_table_{self.rotary_dim}_{self.theta!r}_{self.scaling!r}",
                                  (batch.num_tokens, self.rotary_dim // 2, 2), torch.float32)
             table = batch.shared[key] = ops.rope_table(batch.positions, self.inv_freq, out=out)
         return table
