@@ -408,11 +408,31 @@ def dedelorn_shape(size, layers, vocab):
     return dict(architecture="Dedelorn", width=z["width"], vocab=vocab, norm=dict(eps=1e-6), layers=out)
 
 
+def tosisun_shape(size, layers, vocab):
+    """Layer sizes that resemble a real model's, for the Tosisun design: grouped-query attention (as many key/value
+    heads as the Qwen2 model beside it) with heads of 128, four convolution taps, half of every head turned, stretched
+    wavelengths; dense feed-forwards alternate with clamped experts and a shared expert; every fourth layer runs
+    with the tensors of the layer two before it."""
+    z = DESIGN_SIZES[size]
+    out = []
+    for i in range(layers):
+        mixer = dict(heads=z["heads"], kv_heads=max(2, z["heads"] // 7), dim=128, vdim=128, conv=4, scale=128 ** -0.5,
+                     rot=dict(base=500000.0, dims=64, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
+        mlp = dict(kind="dense", ff=z["ff"]) if i % 2 == 0 else \
+            dict(kind="moe", expert=dict(ff=z["expert_ff"], limit=7.0), router=dict(experts=z["experts"], top=z["top"]),
+                 shared=dict(ff=z["expert_ff"], limit=7.0))
+        layer = dict(type="attention", mixer=mixer, mlp=mlp)
+        if i % 4 == 3:
+            layer["weights_of"] = i - 2
+        out.append(layer)
+    return dict(architecture="Tosisun", width=z["width"], vocab=vocab, norm=dict(eps=1e-5), logit_softcap=30.0, layers=out)
+
+
 def design_comparison(args):
     """Prefill and decode of a model of the design at a real model's layer sizes, and of the benchmark's own
     architecture (Qwen2 dense) at the same width, layers, heads and dense feed-forward, one after the other."""
     import torch
-    from zedinfer_amd.config import DedelornConfig, Qwen2Config, SchedulerConfig
+    from zedinfer_amd.config import DedelornConfig, Qwen2Config, SchedulerConfig, TosisunConfig
     from zedinfer_amd.engine import Engine
     layers = args.layers if args.layers != FULL_LAYERS else 8
     vocab, prompt = 32000, args.prompt_len
@@ -420,8 +440,10 @@ def design_comparison(args):
               "data": "synthetic: seeded random weights, seeded uniform-random token ids", "sizes": {}}
     for size in (args.design_sizes.split(",") if args.design_sizes else ["1.5B"]):
         z = DESIGN_SIZES[size]
+        design = {"dedelorn": lambda: (DedelornConfig.from_dict(dedelorn_shape(size, layers, vocab)), "Dedelorn"),
+                  "tosisun": lambda: (TosisunConfig.from_dict(tosisun_shape(size, layers, vocab)), "Tosisun")}[args.design]
         models = {
-            "dedelorn": (DedelornConfig.from_dict(dedelorn_shape(size, layers, vocab)), "Dedelorn"),
+            args.design: design(),
             "qwen2": (Qwen2Config.from_dict(dict(SHAPE, hidden_size=z["width"], intermediate_size=z["ff"], vocab_size=vocab,
                                                  num_hidden_layers=layers, num_attention_heads=z["heads"],
                                                  num_key_value_heads=max(2, z["heads"] // 7), tie_word_embeddings=False)),
@@ -480,7 +502,7 @@ def main():
                     help="run only the 2,048-token prefill (for profiling) and print its figures")
     ap.add_argument("--resident-layer", action="store_true",
                     help="instead: time the one-launch decoder layer (ops.decode_layer) alone, --layers launches a step")
-    ap.add_argument("--design", default="", choices=["", "dedelorn"],
+    ap.add_argument("--design", default="", choices=["", "dedelorn", "tosisun"],
                     help="instead: prefill and decode of a model of this design at a real model's layer sizes, beside "
                          "Qwen2 dense of equal sizes (8 layers unless --layers says otherwise)")
     ap.add_argument("--design-sizes", default="", help="with --design: layer sizes, of " + ", ".join(sorted(DESIGN_SIZES)) +

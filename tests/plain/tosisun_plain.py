@@ -162,12 +162,16 @@ def attention_mixer(cfg, m, w, p: str, x: torch.Tensor) -> torch.Tensor:
     return o.reshape(T, H * dv) @ w[p + "o"].T
 
 
-def feed_forward(cfg, mlp, w, p: str, x: torch.Tensor) -> torch.Tensor:
+def feed_forward(cfg, mlp, w, p: str, x: torch.Tensor, margins=None) -> torch.Tensor:
     if mlp["kind"] == "dense":
         return relu_squared_mlp(x, w[p + "up"], w[p + "down"])
     E, top = int(mlp["router"]["experts"]), int(mlp["router"]["top"])
     limit = float(mlp["expert"]["limit"])
     z = x @ w[p + "router"].T + w[p + "router.b"]
+    if margins is not None and top < E:
+        # how far the last chosen logit lies above the first one left out: a choice within rounding is a close call
+        zs = torch.sort(z, dim=1, descending=True).values
+        margins.append(zs[:, top - 1] - zs[:, top])
     idx, wt = route(z, top)
     out = torch.zeros_like(x)
     for t in range(x.shape[0]):
@@ -180,8 +184,9 @@ def feed_forward(cfg, mlp, w, p: str, x: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def forward(cfg, w, tokens: Sequence[int], return_layers: bool = False):
-    """Logits [T, vocab] of a whole sequence (and the residual stream after every layer)."""
+def forward(cfg, w, tokens: Sequence[int], return_layers: bool = False, margins=None):
+    """Logits [T, vocab] of a whole sequence (and the residual stream after every layer).  ``margins``: a list that
+    receives, for every layer with a router that leaves experts out, each token's margin of the choice [T]."""
     eps = float(cfg["norm"]["eps"])
     x = w["embed"][torch.tensor(list(tokens), dtype=torch.long)]
     after = []
@@ -193,7 +198,7 @@ def forward(cfg, w, tokens: Sequence[int], return_layers: bool = False):
         a = attention_mixer(cfg, layer["mixer"], w, p + "mix.", x)
         x = x + layer_norm(a, w[p + "norm1"], w[p + "norm1.b"], eps)
         if layer.get("mlp") is not None:
-            f = feed_forward(cfg, layer["mlp"], w, p + "mlp.", x)
+            f = feed_forward(cfg, layer["mlp"], w, p + "mlp.", x, margins)
             x = x + layer_norm(f, w[p + "norm2"], w[p + "norm2.b"], eps)
         after.append(x.clone())
     y = layer_norm(x, w["final.norm"], w["final.norm.b"], eps) @ w["head"].T

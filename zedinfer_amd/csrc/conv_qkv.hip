@@ -20,15 +20,24 @@
 #define CQ_MAX_CHANNELS 15360
 #define CQ_MAX_TAPS 16
 
+// One value of the projection: the sum of its `splits` partial sums (split s at proj + s * split_stride), in rising order.
 template <typename TP>
-__device__ __forceinline__ float cq_conv(const TP* __restrict__ proj, int64_t ld, const float* __restrict__ bias,
-                                         const float* __restrict__ conv_w, const float* __restrict__ tail, int t,
-                                         int local, int c, int C, int taps) {
+__device__ __forceinline__ float cq_value(const TP* __restrict__ proj, int64_t ld, int splits, int64_t split_stride,
+                                          int64_t row, int c) {
+    float v = zi_load(proj + row * ld + c);
+    for (int s = 1; s < splits; ++s) v += zi_load(proj + s * split_stride + row * ld + c);
+    return v;
+}
+
+template <typename TP>
+__device__ __forceinline__ float cq_conv(const TP* __restrict__ proj, int64_t ld, int splits, int64_t split_stride,
+                                         const float* __restrict__ bias, const float* __restrict__ conv_w,
+                                         const float* __restrict__ tail, int t, int local, int c, int C, int taps) {
     float y = 0.f;
     const float bc = bias ? bias[c] : 0.f;
     for (int j = 0; j < taps; ++j) {
         const int li = local - (taps - 1) + j;
-        const float u = li >= 0 ? zi_load(proj + (int64_t)(t - local + li) * ld + c) + bc
+        const float u = li >= 0 ? cq_value(proj, ld, splits, split_stride, t - local + li, c) + bc
                                 : tail[(int64_t)(li + taps - 1) * C + c];
         y += conv_w[(int64_t)c * taps + j] * u;
     }
@@ -38,8 +47,9 @@ __device__ __forceinline__ float cq_conv(const TP* __restrict__ proj, int64_t ld
 template <typename TP, typename T>
 __global__ void __launch_bounds__(CQ_THREADS)
 conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* __restrict__ vcache,
-                const TP* __restrict__ proj, int64_t ld, const float* __restrict__ bias, const float* __restrict__ conv_w,
-                const float* __restrict__ state, int64_t state_stride, const float* __restrict__ q_norm,
+                const TP* __restrict__ proj, int64_t ld, int splits, int64_t split_stride, const float* __restrict__ bias,
+                const float* __restrict__ conv_w, float* __restrict__ state, int64_t state_stride, int move_tail,
+                const float* __restrict__ q_norm,
                 const float* __restrict__ k_norm, float eps, const float* __restrict__ table, int rot,
                 const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ entry_start,
                 const int32_t* __restrict__ entry_slot, const int32_t* __restrict__ slots, int64_t cache_slots, int nh,
@@ -48,13 +58,21 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
     __shared__ float red[16];
     const int t = blockIdx.x, e = tok_seq[t], local = t - entry_start[e];
     const int Qd = nh * dim, Kd = nkv * dim, Vd = nkv * vdim, C = Qd + Kd + Vd;
-    const float* tail = state + (int64_t)entry_slot[e] * state_stride;
+    float* tail = state + (int64_t)entry_slot[e] * state_stride;
+    const int slot = slots ? slots[t] : -1;
     float sq = 0.f, sk = 0.f;
     for (int c = threadIdx.x; c < C; c += CQ_THREADS) {
-        const float v = cq_conv(proj, ld, bias, conv_w, tail, t, local, c, C, taps);
+        const float v = cq_conv(proj, ld, splits, split_stride, bias, conv_w, tail, t, local, c, C, taps);
         y[c] = v;
         if (c < Qd) sq += v * v;
         else if (c < Qd + Kd) sk += v * v;
+        // a step in which every entry brings one token: no other workgroup reads this entry's tail, and this thread
+        // alone reads and writes channel c of it, so the tail moves on here (a token without a place in the cache is
+        // padding and moves nothing)
+        if (move_tail && slot >= 0 && taps > 1) {
+            for (int k = 0; k + 2 < taps; ++k) tail[(int64_t)k * C + c] = tail[(int64_t)(k + 1) * C + c];
+            tail[(int64_t)(taps - 2) * C + c] = cq_value(proj, ld, splits, split_stride, t, c) + (bias ? bias[c] : 0.f);
+        }
     }
     sq = zi_block_sum(sq, red);
     sk = zi_block_sum(sk, red);
@@ -79,8 +97,7 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
         }
         zi_store(q_out + (int64_t)t * ldq + i, v);
     }
-    const int slot = slots ? slots[t] : -1;
-    if (slot < 0 || (int64_t)slot >= cache_slots) return;      // a token without a place in the cache stores nothing
+    if (!kcache || slot < 0 || (int64_t)slot >= cache_slots) return;      // a token without a place in the cache stores nothing
     const int64_t page = slot / page_size, off = slot % page_size;
     for (int i = threadIdx.x; i < nkv * D; i += CQ_THREADS) {
         const int g = i / D, x = i % D;
@@ -105,9 +122,12 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
     }
 }
 
+// `move_tail` (only for steps in which every entry brings one token): the kernel also writes the new tail, and
+// zi_conv_tail is not needed.  `splits` > 1: proj comes as float32 partial sums [splits][n][ld].
 extern "C" int zi_conv_qkv(void* q_out, int dt, int64_t ldq, void* kcache, void* vcache, const void* proj, int proj_dt,
-                           int64_t ld, const float* bias, const float* conv_w, const float* state, int64_t state_stride,
-                           const float* q_norm, const float* k_norm, float eps, const float* table, int rot, int n,
+                           int64_t ld, int splits, int64_t split_stride, const float* bias, const float* conv_w,
+                           float* state, int64_t state_stride, int move_tail, const float* q_norm, const float* k_norm,
+                           float eps, const float* table, int rot, int n,
                            const int32_t* tok_seq, const int32_t* entry_start, const int32_t* entry_slot,
                            const int32_t* slots, int64_t cache_slots, int nh, int nkv, int dim, int vdim, int D, int taps,
                            int page_size, hipStream_t stream) {
@@ -120,12 +140,15 @@ extern "C" int zi_conv_qkv(void* q_out, int dt, int64_t ldq, void* kcache, void*
     ZI_REQUIRE(state_stride >= (int64_t)(taps - 1) * C, "conv_qkv: the state row is too short");
     ZI_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dim && (rot == 0 || table), "conv_qkv: %d rotated dims of %d", rot, dim);
     ZI_REQUIRE(eps > 0.f, "conv_qkv: eps must be positive");
-    ZI_REQUIRE(!slots || (kcache && vcache && cache_slots > 0), "conv_qkv: slots without a cache");
+    ZI_REQUIRE(!(kcache || vcache) || (slots && kcache && vcache && cache_slots > 0), "conv_qkv: a cache without slots");
+    ZI_REQUIRE(splits >= 1 && (splits == 1 || proj_dt == ZI_F32), "conv_qkv: partial sums are float32");
+    ZI_REQUIRE(!move_tail || slots, "conv_qkv: moving the tail needs the tokens' slots");
     if (n == 0) return 0;
     const size_t lds = (size_t)C * sizeof(float);
     ZI_DISPATCH_DTYPE(proj_dt, TP, ZI_DISPATCH_DTYPE(dt, T, {
         conv_qkv_kernel<TP, T><<<n, CQ_THREADS, lds, stream>>>(
-            (T*)q_out, ldq, (T*)kcache, (T*)vcache, (const TP*)proj, ld, bias, conv_w, state, state_stride, q_norm, k_norm,
+            (T*)q_out, ldq, (T*)kcache, (T*)vcache, (const TP*)proj, ld, splits, split_stride, bias, conv_w, state,
+            state_stride, move_tail, q_norm, k_norm,
             eps, table, rot, tok_seq, entry_start, entry_slot, slots, cache_slots, nh, nkv, dim, vdim, D, taps, page_size);
     }));
     return zi_check_launch("conv_qkv");
@@ -133,15 +156,29 @@ extern "C" int zi_conv_qkv(void* q_out, int dt, int64_t ldq, void* kcache, void*
 
 // The convolution's new tail: the last taps - 1 rows of u = projection + bias of the sequence so far, from this
 // step's rows and, where the entry brought fewer, from the old tail.  A thread reads all it needs of the old tail
-// before it writes.
+// before it writes.  With `slots` (every token's place in the cache, negative for tokens that have none), only an
+// entry's own tokens count: those without a place stand behind them (padding that gives steps recurring shapes) and
+// must not move the tail, and an entry that has none at all (it belongs to no request) leaves its slot's tail alone.
 template <typename TP>
 __global__ void __launch_bounds__(256)
-conv_tail_kernel(float* __restrict__ state, int64_t state_stride, const TP* __restrict__ proj, int64_t ld,
-                 const float* __restrict__ bias, const int32_t* __restrict__ entry_start,
-                 const int32_t* __restrict__ entry_len, const int32_t* __restrict__ entry_slot, int C, int taps) {
+conv_tail_kernel(float* __restrict__ state, int64_t state_stride, const TP* __restrict__ proj, int64_t ld, int splits,
+                 int64_t split_stride, const float* __restrict__ bias, const int32_t* __restrict__ entry_start,
+                 const int32_t* __restrict__ entry_len, const int32_t* __restrict__ entry_slot,
+                 const int32_t* __restrict__ slots, int C, int taps) {
     const int e = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
     if (c >= C) return;
-    const int start = entry_start[e], len = entry_len[e];
+    const int start = entry_start[e];
+    int len = entry_len[e];
+    if (slots) {
+        int lo = 0, hi = len;          // the first token without a place: the entry's own tokens come first
+        while (lo < hi) {
+            const int mid = (lo + hi) / 2;
+            if (slots[start + mid] >= 0) lo = mid + 1;
+            else hi = mid;
+        }
+        len = lo;
+        if (len == 0) return;
+    }
     float* tail = state + (int64_t)entry_slot[e] * state_stride;
     const float bc = bias ? bias[c] : 0.f;
     float keep[CQ_MAX_TAPS];
@@ -149,7 +186,7 @@ conv_tail_kernel(float* __restrict__ state, int64_t state_stride, const TP* __re
     for (int k = 0; k < CQ_MAX_TAPS; ++k) {
         if (k >= taps - 1) break;
         const int li = len - (taps - 1) + k;
-        keep[k] = li >= 0 ? zi_load(proj + (int64_t)(start + li) * ld + c) + bc : tail[(int64_t)(li + taps - 1) * C + c];
+        keep[k] = li >= 0 ? cq_value(proj, ld, splits, split_stride, start + li, c) + bc : tail[(int64_t)(li + taps - 1) * C + c];
     }
 #pragma unroll
     for (int k = 0; k < CQ_MAX_TAPS; ++k) {
@@ -158,16 +195,19 @@ conv_tail_kernel(float* __restrict__ state, int64_t state_stride, const TP* __re
     }
 }
 
-extern "C" int zi_conv_tail(float* state, int64_t state_stride, const void* proj, int proj_dt, int64_t ld,
-                            const float* bias, const int32_t* entry_start, const int32_t* entry_len,
-                            const int32_t* entry_slot, int entries, int channels, int taps, hipStream_t stream) {
+extern "C" int zi_conv_tail(float* state, int64_t state_stride, const void* proj, int proj_dt, int64_t ld, int splits,
+                            int64_t split_stride, const float* bias, const int32_t* entry_start, const int32_t* entry_len,
+                            const int32_t* entry_slot, const int32_t* slots, int entries, int channels, int taps,
+                            hipStream_t stream) {
     ZI_REQUIRE(entries >= 0 && entries <= 65535 && channels > 0 && taps >= 1 && taps <= CQ_MAX_TAPS,
                "conv_tail: bad sizes (at most %d taps)", CQ_MAX_TAPS);
     ZI_REQUIRE(ld >= channels && state_stride >= (int64_t)(taps - 1) * channels, "conv_tail: a row is too short");
+    ZI_REQUIRE(splits >= 1 && (splits == 1 || proj_dt == ZI_F32), "conv_tail: partial sums are float32");
     if (entries == 0 || taps == 1) return 0;
     ZI_DISPATCH_DTYPE(proj_dt, TP, {
         conv_tail_kernel<TP><<<dim3((channels + 255) / 256, entries), 256, 0, stream>>>(
-            state, state_stride, (const TP*)proj, ld, bias, entry_start, entry_len, entry_slot, channels, taps);
+            state, state_stride, (const TP*)proj, ld, splits, split_stride, bias, entry_start, entry_len, entry_slot, slots,
+            channels, taps);
     });
     return zi_check_launch("conv_tail");
 }

@@ -169,14 +169,15 @@ int zi_layer_norm(void* out, int out_dt, int64_t ldo, float* resid, const void* 
     stream);
 // conv_qkv.hip
 int zi_conv_qkv(void* q_out, int dt, int64_t ldq, void* kcache, void* vcache, const void* proj, int proj_dt, int64_t ld,
-    const float* bias, const float* conv_w, const float* state, int64_t state_stride, const float* q_norm, const float*
-    k_norm, float eps, const float* table, int rot, int n, const int32_t* tok_seq, const int32_t* entry_start, const
+    int splits, int64_t split_stride, const float* bias, const float* conv_w, float* state, int64_t state_stride, int
+    move_tail, const float* q_norm, const float* k_norm, float eps, const float* table, int rot, int n, const int32_t* tok_seq, const int32_t* entry_start, const
     int32_t* entry_slot, const int32_t* slots, int64_t cache_slots, int nh, int nkv, int dim, int vdim, int D, int taps,
     int page_size, hipStream_t stream);
 // conv_qkv.hip
-int zi_conv_tail(float* state, int64_t state_stride, const void* proj, int proj_dt, int64_t ld, const float* bias, const
-    int32_t* entry_start, const int32_t* entry_len, const int32_t* entry_slot, int entries, int channels, int taps,
-    hipStream_t stream);
+int zi_conv_tail(float* state, int64_t state_stride, const void* proj, int proj_dt, int64_t ld, int splits, int64_t
+    split_stride, const float* bias, const
+    int32_t* entry_start, const int32_t* entry_len, const int32_t* entry_slot, const int32_t* slots, int entries, int
+    channels, int taps, hipStream_t stream);
 // elementwise.hip
 int zi_relu_squared(void* out, int out_dt, int64_t ldo, const void* z, int dt, int64_t ldz, int splits, int64_t
     split_stride, int n, int inter, hipStream_t stream);

@@ -65,17 +65,19 @@ def conv_qkv(proj: torch.Tensor, bias: Optional[torch.Tensor], conv_w: torch.Ten
              q_norm: torch.Tensor, k_norm: torch.Tensor, eps: float, table: Optional[torch.Tensor], tok_seq: torch.Tensor,
              entry_start: torch.Tensor, entry_slot: torch.Tensor, slots: Optional[torch.Tensor],
              kcache: Optional[torch.Tensor], vcache: Optional[torch.Tensor], nh: int, nkv: int, dim: int, vdim: int,
-             head: int, taps: int, q_out: torch.Tensor) -> torch.Tensor:
-    """Rows of proj [n, nh*dim + nkv*dim + nkv*vdim] (q | k | v, any storage type) plus ``bias`` pass, per channel, a
+             head: int, taps: int, q_out: torch.Tensor, move_tail: bool = False) -> torch.Tensor:
+    """Rows of proj [n, nh*dim + nkv*dim + nkv*vdim] (q | k | v, any storage type, or a stack [S, n, ...] of float32
+    partial sums) plus ``bias`` pass, per channel, a
     causal convolution of ``taps`` taps (``conv_w`` [channels, taps]; rows before the step come from the request's
     tail in ``state`` [slots, >= (taps-1) * channels]), q and k an RMS norm over all their channels at once (gains
     ``q_norm`` / ``k_norm``), and a split-half rotation of the first R dims of every head by ``table`` [n, R/2, 2].
-    The queries go to ``q_out`` [n, nh*head]; keys and values, where ``slots`` is given, into the paged cache whose
-    heads hold ``head`` >= dim, vdim values (the rest zero).  Everything float32 but the stores."""
+    The queries go to ``q_out`` [n, nh*head]; keys and values, where the caches are given, into the paged cache at
+    ``slots`` (a token whose slot is negative stores nothing), whose heads hold ``head`` >= dim, vdim values (the
+    rest zero).  ``move_tail`` (only when every entry brings one token): the new tails are written here too, for
+    tokens that have a slot, and ``conv_tail`` is not needed.  Everything float32 but the stores."""
     _gpu("conv_qkv", proj, bias, conv_w, state, q_norm, k_norm, table, tok_seq, entry_start, entry_slot, slots, kcache,
          vcache, q_out)
-    ld, width = _rows(proj, "conv_qkv proj")
-    n = proj.shape[0]
+    splits, split_stride, ld, n, width = _terms(proj, "conv_qkv proj")
     Qd, Kd, Vd = nh * dim, nkv * dim, nkv * vdim
     C = Qd + Kd + Vd
     if width != C:
@@ -103,21 +105,31 @@ def conv_qkv(proj: torch.Tensor, bias: Optional[torch.Tensor], conv_w: torch.Ten
         raise ValueError(f"conv_qkv: q_out must be [n, {nh * head}] with heads of at least {max(dim, vdim)} values")
     pages = ps = 0
     if slots is not None:
-        pages, ps = _check_cache(kcache, vcache, nkv, head, q_out.dtype, "conv_qkv")
         _i32(slots, "conv_qkv slots", n)
-    _lib.call("zi_conv_qkv", _p(q_out), _code(q_out, "conv_qkv q_out"), ldq, _p(kcache if slots is not None else None),
-              _p(vcache if slots is not None else None), _p(proj), _code(proj, "conv_qkv proj"), ld, _p(bias), _p(conv_w),
-              _p(state), int(state.stride(0)), _p(q_norm), _p(k_norm), float(eps), _p(table), rot, n, _p(tok_seq),
+    if kcache is not None:
+        if slots is None:
+            raise ValueError("conv_qkv: a cache needs the tokens' slots")
+        pages, ps = _check_cache(kcache, vcache, nkv, head, q_out.dtype, "conv_qkv")
+    if move_tail and slots is None:
+        raise ValueError("conv_qkv: moving the tail needs the tokens' slots")
+    _lib.call("zi_conv_qkv", _p(q_out), _code(q_out, "conv_qkv q_out"), ldq, _p(kcache),
+              _p(vcache if kcache is not None else None), _p(proj), _code(proj, "conv_qkv proj"), ld, splits, split_stride,
+              _p(bias), _p(conv_w), _p(state), int(state.stride(0)), int(bool(move_tail)), _p(q_norm), _p(k_norm),
+              float(eps), _p(table), rot, n, _p(tok_seq),
               _p(entry_start), _p(entry_slot), _p(slots), pages * ps, nh, nkv, dim, vdim, head, taps, max(ps, 1), _stream())
     return q_out
 
 
 def conv_tail(state: torch.Tensor, proj: torch.Tensor, bias: Optional[torch.Tensor], entry_start: torch.Tensor,
-              entry_len: torch.Tensor, entry_slot: torch.Tensor, taps: int) -> None:
+              entry_len: torch.Tensor, entry_slot: torch.Tensor, taps: int, slots: Optional[torch.Tensor] = None) -> None:
     """After ``conv_qkv`` has read the old tails: the last taps - 1 rows of proj + bias of every entry's sequence so
-    far become the new tail in the entry's state slot."""
-    _gpu("conv_tail", state, proj, bias, entry_start, entry_len, entry_slot)
-    ld, C = _rows(proj, "conv_tail proj")
+    far become the new tail in the entry's state slot.  With ``slots`` (every token's place in the cache) the tokens
+    that have none (negative; they stand behind an entry's own) do not count, and an entry without any token of its
+    own leaves its slot's tail as it is."""
+    _gpu("conv_tail", state, proj, bias, entry_start, entry_len, entry_slot, slots)
+    splits, split_stride, ld, n, C = _terms(proj, "conv_tail proj")
+    if slots is not None:
+        _i32(slots, "conv_tail slots", n)
     if state.dtype != torch.float32 or state.dim() != 2 or not state.is_contiguous() or state.shape[1] < (taps - 1) * C:
         raise ValueError(f"conv_tail: state must be contiguous float32 [slots, >= {(taps - 1) * C}]")
     if bias is not None:
@@ -127,8 +139,9 @@ def conv_tail(state: torch.Tensor, proj: torch.Tensor, bias: Optional[torch.Tens
         _i32(t, f"conv_tail {name}", E)
     if not (1 <= taps <= CONV_MAX_TAPS):
         raise ValueError(f"conv_tail: at most {CONV_MAX_TAPS} taps")
-    _lib.call("zi_conv_tail", _p(state), int(state.stride(0)), _p(proj), _code(proj, "conv_tail proj"), ld, _p(bias),
-              _p(entry_start), _p(entry_len), _p(entry_slot), E, C, taps, _stream())
+    _lib.call("zi_conv_tail", _p(state), int(state.stride(0)), _p(proj), _code(proj, "conv_tail proj"), ld, splits,
+              split_stride, _p(bias),
+              _p(entry_start), _p(entry_len), _p(entry_slot), _p(slots), E, C, taps, _stream())
 
 
 def relu_squared(z: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
@@ -145,8 +158,16 @@ def relu_squared(z: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 
 def clamped_glu(gate: torch.Tensor, up: torch.Tensor, limit: float, out: torch.Tensor, alpha: float = 1.702) -> torch.Tensor:
     """out = g sigmoid(alpha g) (u + 1) with g = min(gate, limit), u = clamp(up, -limit, limit); gate and up [n, I]
-    with dense rows (column slices of one product are fine)."""
+    with dense rows (column slices of one product are fine), or the same slices [S, n, I] of a stack of float32 partial
+    sums, which are added first."""
     _gpu("clamped_glu", gate, up, out)
+    splits, split_stride = 1, 0
+    if gate.dim() == 3:
+        if gate.dtype != torch.float32 or up.dtype != torch.float32 or gate.shape != up.shape or gate.stride() != up.stride() \
+                or gate.stride(2) != 1:
+            raise ValueError("clamped_glu: stacks of partial sums must be float32 slices of one stack")
+        splits, split_stride = int(gate.shape[0]), int(gate.stride(0))
+        gate, up = gate[0], up[0]
     ldg, I = _rows(gate, "clamped_glu gate")
     ldu, Iu = _rows(up, "clamped_glu up")
     ldo, Io = _rows(out, "clamped_glu out")
@@ -156,7 +177,7 @@ def clamped_glu(gate: torch.Tensor, up: torch.Tensor, limit: float, out: torch.T
     if not limit > 0:
         raise ValueError("clamped_glu: the limit must be positive")
     _lib.call("zi_clamped_glu", _p(out), _code(out, "clamped_glu out"), ldo, _p(gate), _p(up), _code(gate, "clamped_glu"),
-              ldg, ldu, 1, 0, n, I, float(limit), float(alpha), _stream())
+              ldg, ldu, splits, split_stride, n, I, float(limit), float(alpha), _stream())
     return out
 
 

@@ -294,8 +294,9 @@ class Mixer(Part):
     # place in the cache (slot -1), whose results nobody reads; and it may add entries of one such token
     # that belong to no request (state slot 0, an empty block table).  A mixer for which that changes
     # nothing any real token sees sets this; one that keeps state per request must leave it False, or
-    # the padding would advance its state.  One mixer that leaves it False keeps the whole model's steps
-    # unpadded.
+    # the padding would advance its state (unless its kernels tell the padding by its missing slot and
+    # leave the state of such tokens and entries alone, as the attention with convolved projections
+    # does).  One mixer that leaves it False keeps the whole model's steps unpadded.
     padding_safe: bool = False
 
     def planner(self) -> Optional[StepPlanner]:

@@ -350,9 +350,14 @@ class _ClampedGated:
 
     def forward(self, rt: Runtime, x: torch.Tensor, name: str) -> torch.Tensor:
         n, I = x.shape[0], self.inter
-        gu = ops.linear(x, self.gate_up, out=rt.buffer(name + "_gate_up", (n, self.up_at + I), torch.float32))
         act = rt.buffer(name + "_act", (n, I))
-        ops.clamped_glu(gu[:, :I], gu[:, self.up_at:], self.limit, out=act)
+        if ops.linear_sums_supported(x, self.gate_up):
+            S = ops.linear_splits(n, self.up_at + I, self.hidden)
+            gu = ops.linear_sums(x, self.gate_up, out=rt.buffer(name + "_gate_up_sums", (S, n, self.up_at + I), torch.float32))
+            ops.clamped_glu(gu[:, :, :I], gu[:, :, self.up_at:], self.limit, out=act)
+        else:
+            gu = ops.linear(x, self.gate_up, out=rt.buffer(name + "_gate_up", (n, self.up_at + I), torch.float32))
+            ops.clamped_glu(gu[:, :I], gu[:, self.up_at:], self.limit, out=act)
         return act
 
 

@@ -404,11 +404,13 @@ class ConvAttention(Attention):
     output, and W_o gets zero columns where the padding stands.  A request's state is the last conv - 1 rows that
     entered the convolution (float32, the biases in them).  Everything between the projection and the attention
     kernels is one launch in float32 arithmetic (``csrc/conv_qkv.hip``); the projections leave float32 results.
-    Steps of such a model are never padded: a padding token would move the convolution's tail.
+    Steps may be padded although the mixer keeps state: a padding token has no place in the cache, the kernel that
+    writes the new tail counts only the tokens that have one, and an entry of no request leaves the tail of the slot
+    it names alone.
 
     params: hidden_size, num_heads, num_kv_heads, head_dim, value_dim, conv, scale, window (0), eps, position."""
 
-    padding_safe = False
+    padding_safe = True
 
     @staticmethod
     def weight_specs(spec: PartSpec) -> Dict[str, WeightSpec]:
@@ -481,14 +483,23 @@ class ConvAttention(Attention):
         table = self.position.step_table(batch)
         if table is None:
             raise ValueError("conv_attention: the position encoding must hand over a table of split-half angles")
-        proj = ops.linear(x, self.qkv, out=rt.buffer("conv_attn_proj", (n, self.channels), torch.float32))
+        if ops.linear_sums_supported(x, self.qkv):
+            # few rows: the projection leaves float32 partial sums, which the next kernel adds as it reads them
+            S = ops.linear_splits(n, self.channels, self.hidden)
+            proj = ops.linear_sums(x, self.qkv, out=rt.buffer("conv_attn_sums", (S, n, self.channels), torch.float32))
+        else:
+            proj = ops.linear(x, self.qkv, out=rt.buffer("conv_attn_proj", (n, self.channels), torch.float32))
         q = rt.buffer("attn_q", (n, self.qd))
         writes = memory.writes
+        # when every entry brings one token, the kernel that reads a tail is the only one that does, and moves it on
+        single = bool(batch.single_tokens)
         ops.conv_qkv(proj, self.bias, self.conv_w, memory.state, self.q_norm, self.k_norm, self.eps,
                      None if isinstance(table, str) else table, batch.tok_seq, batch.entry_start, batch.entry_slot,
-                     view.slots if writes else None, memory.tensors["k"] if writes else None,
-                     memory.tensors["v"] if writes else None, self.nh, self.nkv, self.dim, self.vdim, self.d, self.taps, q)
-        ops.conv_tail(memory.state, proj, self.bias, batch.entry_start, batch.entry_len, batch.entry_slot, self.taps)
+                     view.slots, memory.tensors["k"] if writes else None, memory.tensors["v"] if writes else None,
+                     self.nh, self.nkv, self.dim, self.vdim, self.d, self.taps, q, move_tail=single)
+        if not single:
+            ops.conv_tail(memory.state, proj, self.bias, batch.entry_start, batch.entry_len, batch.entry_slot, self.taps,
+                          slots=view.slots)
         att = rt.buffer("attn_out", (n, self.qd))
         self.attend(q, att, batch, view, memory)
         return self.project(att, n)
