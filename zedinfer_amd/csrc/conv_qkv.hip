@@ -29,13 +29,40 @@ __device__ __forceinline__ float cq_value(const TP* __restrict__ proj, int64_t l
     return v;
 }
 
-template <typename TP>
+// The convolved value of channel c of token t; `now` receives the token's own input (projection + bias).  With the
+// number of taps known at compile time (TAPS > 0) and float32 rows that are no partial sums, every tap's input is one
+// load whose address alone depends on where it comes from (the projection or the tail), so all are in flight together.
+template <typename TP, int TAPS>
 __device__ __forceinline__ float cq_conv(const TP* __restrict__ proj, int64_t ld, int splits, int64_t split_stride,
                                          const float* __restrict__ bias, const float* __restrict__ conv_w,
-                                         const float* __restrict__ tail, int t, int local, int c, int C, int taps) {
-    float y = 0.f;
+                                         const float* __restrict__ tail, int t, int local, int c, int C, int taps,
+                                         float& now) {
     const float bc = bias ? bias[c] : 0.f;
-    for (int j = 0; j < taps; ++j) {
+    if constexpr (TAPS > 0 && sizeof(TP) == 4) {
+        if (splits == 1) {
+            float u[TAPS], wv[TAPS];
+#pragma unroll
+            for (int j = 0; j < TAPS; ++j) {
+                const int li = local - (TAPS - 1) + j;
+                const float* src = li >= 0 ? (const float*)proj + (int64_t)(t - local + li) * ld + c
+                                           : tail + (int64_t)(li + TAPS - 1) * C + c;
+                u[j] = *src;
+                wv[j] = conv_w[(int64_t)c * TAPS + j];
+            }
+            float y = 0.f;
+#pragma unroll
+            for (int j = 0; j < TAPS; ++j) {
+                const int li = local - (TAPS - 1) + j;
+                if (li >= 0) u[j] += bc;
+                y += wv[j] * u[j];
+            }
+            now = u[TAPS - 1];
+            return y;
+        }
+    }
+    now = cq_value(proj, ld, splits, split_stride, t, c) + bc;
+    float y = conv_w[(int64_t)c * taps + taps - 1] * now;
+    for (int j = 0; j + 1 < taps; ++j) {
         const int li = local - (taps - 1) + j;
         const float u = li >= 0 ? cq_value(proj, ld, splits, split_stride, t - local + li, c) + bc
                                 : tail[(int64_t)(li + taps - 1) * C + c];
@@ -44,8 +71,8 @@ __device__ __forceinline__ float cq_conv(const TP* __restrict__ proj, int64_t ld
     return y;
 }
 
-template <typename TP, typename T>
-__global__ void __launch_bounds__(CQ_THREADS)
+template <typename TP, typename T, int TAPS, int THREADS>
+__global__ void __launch_bounds__(THREADS)
 conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* __restrict__ vcache,
                 const TP* __restrict__ proj, int64_t ld, int splits, int64_t split_stride, const float* __restrict__ bias,
                 const float* __restrict__ conv_w, float* __restrict__ state, int64_t state_stride, int move_tail,
@@ -61,8 +88,9 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
     float* tail = state + (int64_t)entry_slot[e] * state_stride;
     const int slot = slots ? slots[t] : -1;
     float sq = 0.f, sk = 0.f;
-    for (int c = threadIdx.x; c < C; c += CQ_THREADS) {
-        const float v = cq_conv(proj, ld, splits, split_stride, bias, conv_w, tail, t, local, c, C, taps);
+    for (int c = threadIdx.x; c < C; c += THREADS) {
+        float now;
+        const float v = cq_conv<TP, TAPS>(proj, ld, splits, split_stride, bias, conv_w, tail, t, local, c, C, taps, now);
         y[c] = v;
         if (c < Qd) sq += v * v;
         else if (c < Qd + Kd) sk += v * v;
@@ -71,7 +99,7 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
         // padding and moves nothing)
         if (move_tail && slot >= 0 && taps > 1) {
             for (int k = 0; k + 2 < taps; ++k) tail[(int64_t)k * C + c] = tail[(int64_t)(k + 1) * C + c];
-            tail[(int64_t)(taps - 2) * C + c] = cq_value(proj, ld, splits, split_stride, t, c) + (bias ? bias[c] : 0.f);
+            tail[(int64_t)(taps - 2) * C + c] = now;
         }
     }
     sq = zi_block_sum(sq, red);
@@ -81,7 +109,7 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
     const int half = rot / 2;
     const float* ang = table ? table + (int64_t)t * half * 2 : nullptr;
     // queries: every (head, dim of the padded head)
-    for (int i = threadIdx.x; i < nh * D; i += CQ_THREADS) {
+    for (int i = threadIdx.x; i < nh * D; i += THREADS) {
         const int h = i / D, x = i % D;
         float v = 0.f;
         if (x < dim) {
@@ -99,7 +127,7 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
     }
     if (!kcache || slot < 0 || (int64_t)slot >= cache_slots) return;      // a token without a place in the cache stores nothing
     const int64_t page = slot / page_size, off = slot % page_size;
-    for (int i = threadIdx.x; i < nkv * D; i += CQ_THREADS) {
+    for (int i = threadIdx.x; i < nkv * D; i += THREADS) {
         const int g = i / D, x = i % D;
         float v = 0.f;
         if (x < dim) {
@@ -115,7 +143,7 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
         }
         zi_store(kcache + ((page * nkv + g) * page_size + off) * D + x, v);
     }
-    for (int i = threadIdx.x; i < nkv * D; i += CQ_THREADS) {
+    for (int i = threadIdx.x; i < nkv * D; i += THREADS) {
         const int g = i / D, x = i % D;
         const float v = x < vdim ? y[Qd + Kd + g * vdim + x] : 0.f;
         zi_store(vcache + ((page * nkv + g) * D + x) * page_size + off, v);
@@ -145,12 +173,25 @@ extern "C" int zi_conv_qkv(void* q_out, int dt, int64_t ldq, void* kcache, void*
     ZI_REQUIRE(!move_tail || slots, "conv_qkv: moving the tail needs the tokens' slots");
     if (n == 0) return 0;
     const size_t lds = (size_t)C * sizeof(float);
+    // few tokens: workgroups of 1,024 threads, so that a thread walks few channels one after the other
+    const bool wide = n <= 512 && C > CQ_THREADS;
+#define ZI_CQ(TAPS, THREADS)                                                                                           \
+    conv_qkv_kernel<TP, T, TAPS, THREADS><<<n, THREADS, lds, stream>>>(                                                \
+        (T*)q_out, ldq, (T*)kcache, (T*)vcache, (const TP*)proj, ld, splits, split_stride, bias, conv_w, state,       \
+        state_stride, move_tail, q_norm, k_norm, eps, table, rot, tok_seq, entry_start, entry_slot, slots, cache_slots, \
+        nh, nkv, dim, vdim, D, taps, page_size)
+#define ZI_CQ_TAPS(THREADS)                                                 \
+    switch (taps) {                                                         \
+        case 2: ZI_CQ(2, THREADS); break;                                   \
+        case 3: ZI_CQ(3, THREADS); break;                                   \
+        case 4: ZI_CQ(4, THREADS); break;                                   \
+        default: ZI_CQ(0, THREADS); break;                                  \
+    }
     ZI_DISPATCH_DTYPE(proj_dt, TP, ZI_DISPATCH_DTYPE(dt, T, {
-        conv_qkv_kernel<TP, T><<<n, CQ_THREADS, lds, stream>>>(
-            (T*)q_out, ldq, (T*)kcache, (T*)vcache, (const TP*)proj, ld, splits, split_stride, bias, conv_w, state,
-            state_stride, move_tail, q_norm, k_norm,
-            eps, table, rot, tok_seq, entry_start, entry_slot, slots, cache_slots, nh, nkv, dim, vdim, D, taps, page_size);
+        if (wide) { ZI_CQ_TAPS(1024) } else { ZI_CQ_TAPS(CQ_THREADS) }
     }));
+#undef ZI_CQ_TAPS
+#undef ZI_CQ
     return zi_check_launch("conv_qkv");
 }
 

@@ -238,6 +238,54 @@ extern "C" int zi_gated_act(void* out, int out_dt, int64_t ldo, const void* gate
 }
 
 // ---- activations of feed-forwards without the SiLU gate ------------------------------------------------------
+// Four consecutive values at a time where rows allow it (widths and strides multiples of four, 16-byte aligned).
+__device__ __forceinline__ float4 ew_load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 ew_load4(const zi_bf16* p) {
+    const uint2 r = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
+                       __uint_as_float(r.y & 0xffff0000u));
+}
+__device__ __forceinline__ void ew_store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void ew_store4(zi_bf16* p, float4 v) {
+    uint2 r;
+    r.x = zi_pack_bf16x2(v.x, v.y);
+    r.y = zi_pack_bf16x2(v.z, v.w);
+    *reinterpret_cast<uint2*>(p) = r;
+}
+static bool ew_rows4(const void* p, int64_t ld, int inter) {
+    return inter % 4 == 0 && ld % 4 == 0 && ((uintptr_t)p % 16) == 0;
+}
+
+template <typename T, typename TO>
+__global__ void relu_squared_vec_kernel(TO* __restrict__ out, int64_t ldo, const T* __restrict__ z, int64_t ldz, int n,
+                                        int inter) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int q = inter / 4;
+    if (i >= (int64_t)n * q) return;
+    const int64_t r = i / q, c = (i % q) * 4;
+    float4 v = ew_load4(z + r * ldz + c);
+    v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f); v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f);
+    ew_store4(out + r * ldo + c, make_float4(v.x * v.x, v.y * v.y, v.z * v.z, v.w * v.w));
+}
+
+template <typename T, typename TO>
+__global__ void clamped_glu_vec_kernel(TO* __restrict__ out, int64_t ldo, const T* __restrict__ gate, const T* __restrict__ up,
+                                       int64_t ld_gate, int64_t ld_up, int n, int inter, float limit, float alpha) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int q = inter / 4;
+    if (i >= (int64_t)n * q) return;
+    const int64_t r = i / q, c = (i % q) * 4;
+    const float4 g4 = ew_load4(gate + r * ld_gate + c), u4 = ew_load4(up + r * ld_up + c);
+    const float g[4] = {g4.x, g4.y, g4.z, g4.w}, u[4] = {u4.x, u4.y, u4.z, u4.w};
+    float o[4];
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float gg = fminf(g[k], limit), uu = fminf(fmaxf(u[k], -limit), limit);
+        o[k] = gg / (1.f + expf(-alpha * gg)) * (uu + 1.f);
+    }
+    ew_store4(out + r * ldo + c, make_float4(o[0], o[1], o[2], o[3]));
+}
+
 // relu(z)^2 of every element of a [n][inter] operand with dense rows, which may come as `splits` float32 partial
 // sums (split s at z + s * split_stride, added in rising order first).
 template <typename T, typename TO>
@@ -257,6 +305,13 @@ extern "C" int zi_relu_squared(void* out, int out_dt, int64_t ldo, const void* z
     ZI_REQUIRE(n >= 0 && inter > 0 && ldo >= inter && ldz >= inter && splits >= 1, "relu_squared: bad sizes");
     if (n == 0) return 0;
     const int64_t total = (int64_t)n * inter;
+    if (splits == 1 && ew_rows4(z, ldz, inter) && ew_rows4(out, ldo, inter)) {
+        ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(out_dt, TO, {
+            relu_squared_vec_kernel<T, TO><<<(unsigned)((total / 4 + 255) / 256), 256, 0, stream>>>(
+                (TO*)out, ldo, (const T*)z, ldz, n, inter);
+        }));
+        return zi_check_launch("relu_squared");
+    }
     ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(out_dt, TO, {
         relu_squared_kernel<T, TO><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(
             (TO*)out, ldo, (const T*)z, ldz, splits, split_stride, n, inter);
@@ -292,6 +347,13 @@ extern "C" int zi_clamped_glu(void* out, int out_dt, int64_t ldo, const void* ga
     ZI_REQUIRE(limit > 0.f, "clamped_glu: the limit must be positive, got %g", (double)limit);
     if (n == 0) return 0;
     const int64_t total = (int64_t)n * inter;
+    if (splits == 1 && ew_rows4(gate, ld_gate, inter) && ew_rows4(up, ld_up, inter) && ew_rows4(out, ldo, inter)) {
+        ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(out_dt, TO, {
+            clamped_glu_vec_kernel<T, TO><<<(unsigned)((total / 4 + 255) / 256), 256, 0, stream>>>(
+                (TO*)out, ldo, (const T*)gate, (const T*)up, ld_gate, ld_up, n, inter, limit, alpha);
+        }));
+        return zi_check_launch("clamped_glu");
+    }
     ZI_DISPATCH_DTYPE(dt, T, ZI_DISPATCH_DTYPE(out_dt, TO, {
         clamped_glu_kernel<T, TO><<<(unsigned)((total + 255) / 256), 256, 0, stream>>>(
             (TO*)out, ldo, (const T*)gate, (const T*)up, ld_gate, ld_up, splits, split_stride, n, inter, limit, alpha);

@@ -93,6 +93,125 @@ layer_norm_kernel(TO* __restrict__ out, int64_t ldo, float* __restrict__ resid, 
     }
 }
 
+// ---- rows of H % 4 == 0 values, 16-byte aligned: everything a thread needs is loaded at once, in pieces of four ----
+__device__ __forceinline__ float4 ln_load4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ float4 ln_load4(const zi_bf16* p) {
+    const uint2 r = *reinterpret_cast<const uint2*>(p);
+    return make_float4(__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
+                       __uint_as_float(r.y & 0xffff0000u));
+}
+__device__ __forceinline__ void ln_store4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ void ln_store4(zi_bf16* p, float4 v) {
+    uint2 r;
+    r.x = zi_pack_bf16x2(v.x, v.y);
+    r.y = zi_pack_bf16x2(v.z, v.w);
+    *reinterpret_cast<uint2*>(p) = r;
+}
+
+// Few rows, up to 16 terms: a workgroup per row, a thread owns IT groups of four consecutive values and issues
+// every term's load before the first is used (the few-rows products leave up to a dozen partial sums).
+template <typename TX, typename TW, typename TO, int IT>
+__global__ void layer_norm_vec_kernel(TO* __restrict__ out, int64_t ldo, float* __restrict__ resid, const TX* __restrict__ x,
+                                      int splits, int64_t split_stride, int64_t ldx, const TW* __restrict__ w,
+                                      const TW* __restrict__ b, int H, float eps) {
+    __shared__ float red[16];
+    const int64_t row = blockIdx.x;
+    float4 v[IT];
+    float sum = 0.f;
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int j = (it * blockDim.x + threadIdx.x) * 4;
+        v[it] = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (j >= H) continue;
+        const TX* xr = x + row * ldx + j;
+        float4 d[16];
+#pragma unroll
+        for (int sp = 0; sp < 16; ++sp)
+            d[sp] = (sp < splits) ? ln_load4(xr + (int64_t)sp * split_stride) : make_float4(0.f, 0.f, 0.f, 0.f);
+        float4 t = d[0];
+#pragma unroll
+        for (int sp = 1; sp < 16; ++sp) { t.x += d[sp].x; t.y += d[sp].y; t.z += d[sp].z; t.w += d[sp].w; }
+        v[it] = t;
+        sum += (t.x + t.y) + (t.z + t.w);
+    }
+    const float mean = zi_block_sum(sum, red) / (float)H;
+    float ss = 0.f;
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int j = (it * blockDim.x + threadIdx.x) * 4;
+        if (j >= H) continue;
+        v[it].x -= mean; v[it].y -= mean; v[it].z -= mean; v[it].w -= mean;
+        ss += (v[it].x * v[it].x + v[it].y * v[it].y) + (v[it].z * v[it].z + v[it].w * v[it].w);
+    }
+    const float r = 1.f / sqrtf(zi_block_sum(ss, red) / (float)H + eps);
+#pragma unroll
+    for (int it = 0; it < IT; ++it) {
+        const int j = (it * blockDim.x + threadIdx.x) * 4;
+        if (j >= H) continue;
+        const float4 wv = ln_load4(w + j), bv = ln_load4(b + j);
+        float4 y = make_float4(v[it].x * r * wv.x + bv.x, v[it].y * r * wv.y + bv.y, v[it].z * r * wv.z + bv.z,
+                               v[it].w * r * wv.w + bv.w);
+        if (resid) {
+            const float4 o = ln_load4(resid + row * H + j);
+            y.x += o.x; y.y += o.y; y.z += o.z; y.w += o.w;
+            ln_store4(resid + row * H + j, y);
+        }
+        if (out) ln_store4(out + row * ldo + j, y);
+    }
+}
+
+// Many rows, one or two terms: a wavefront per row, four rows a workgroup, no barrier.  A lane owns NV groups of four
+// consecutive values, 256 values apart (every load instruction of the wavefront reads 1 KB of the row).
+template <typename TX, typename TW, typename TO, int NV>
+__global__ void __launch_bounds__(4 * ZI_WAVE)
+layer_norm_rows_kernel(TO* __restrict__ out, int64_t ldo, float* __restrict__ resid, const TX* __restrict__ x, int splits,
+                       int64_t split_stride, int64_t ldx, const TW* __restrict__ w, const TW* __restrict__ b, int n, int H,
+                       float eps) {
+    const int lane = threadIdx.x & (ZI_WAVE - 1), wave = threadIdx.x / ZI_WAVE;
+    const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+    if (row >= n) return;
+    const TX* xr = x + row * ldx;
+    const int64_t second = splits > 1 ? split_stride : 0;      // one term: read twice, counted once
+    const float twice = splits > 1 ? 1.f : 0.f;
+    float4 v[NV], d[NV], o[NV];
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+        const int j = (c * ZI_WAVE + lane) * 4, jc = j < H ? j : 0;     // past the row: its start again, unused
+        v[c] = ln_load4(xr + jc);
+        d[c] = ln_load4(xr + second + jc);
+        o[c] = resid ? ln_load4(resid + row * H + jc) : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float sum = 0.f;
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+        const int j = (c * ZI_WAVE + lane) * 4;
+        v[c].x += twice * d[c].x; v[c].y += twice * d[c].y; v[c].z += twice * d[c].z; v[c].w += twice * d[c].w;
+        if (j < H) sum += (v[c].x + v[c].y) + (v[c].z + v[c].w);
+    }
+    const float mean = zi_wave_sum(sum) / (float)H;
+    float ss = 0.f;
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+        const int j = (c * ZI_WAVE + lane) * 4;
+        v[c].x -= mean; v[c].y -= mean; v[c].z -= mean; v[c].w -= mean;
+        if (j < H) ss += (v[c].x * v[c].x + v[c].y * v[c].y) + (v[c].z * v[c].z + v[c].w * v[c].w);
+    }
+    const float r = 1.f / sqrtf(zi_wave_sum(ss) / (float)H + eps);
+#pragma unroll
+    for (int c = 0; c < NV; ++c) {
+        const int j = (c * ZI_WAVE + lane) * 4;
+        if (j >= H) continue;
+        const float4 wv = ln_load4(w + j), bv = ln_load4(b + j);
+        float4 y = make_float4(v[c].x * r * wv.x + bv.x, v[c].y * r * wv.y + bv.y, v[c].z * r * wv.z + bv.z,
+                               v[c].w * r * wv.w + bv.w);
+        if (resid) {
+            y.x += o[c].x; y.y += o[c].y; y.z += o[c].z; y.w += o[c].w;
+            ln_store4(resid + row * H + j, y);
+        }
+        if (out) ln_store4(out + row * ldo + j, y);
+    }
+}
+
 extern "C" int zi_layer_norm(void* out, int out_dt, int64_t ldo, float* resid, const void* x, int x_dt, int splits,
                              int64_t split_stride, int64_t ldx, const void* w, const void* b, int w_dt, int n, int hidden,
                              float eps, hipStream_t stream) {
@@ -103,6 +222,43 @@ extern "C" int zi_layer_norm(void* out, int out_dt, int64_t ldo, float* resid, c
     ZI_REQUIRE(eps > 0.f, "layer_norm: eps must be positive");
     ZI_REQUIRE(w && b, "layer_norm: gain and bias are both needed");
     if (n == 0) return 0;
+    const bool aligned = hidden % 4 == 0 && ldx % 4 == 0 && split_stride % 4 == 0 && ((uintptr_t)x % 16) == 0 &&
+                         ((uintptr_t)w % 16) == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)resid % 16) == 0 &&
+                         ((uintptr_t)out % 16) == 0 && ldo % 4 == 0 && (x_dt == ZI_F32 || (ldx % 8 == 0 && ((uintptr_t)x % 8) == 0)) &&
+                         !(x_dt == ZI_BF16 && splits > 1);
+    if (aligned && n >= 64 && splits <= 2 && hidden <= 8192) {
+        const int nv = (hidden + 4 * ZI_WAVE - 1) / (4 * ZI_WAVE);
+        const int wgs = (n + 3) / 4;
+#define ZI_LN_ROWS(NV)                                                                                                \
+    layer_norm_rows_kernel<TX, TW, TO, NV><<<wgs, 4 * ZI_WAVE, 0, stream>>>(                                          \
+        (TO*)out, ldo, resid, (const TX*)x, splits, split_stride, ldx, (const TW*)w, (const TW*)b, n, hidden, eps)
+        ZI_DISPATCH_DTYPE(x_dt, TX, ZI_DISPATCH_DTYPE(w_dt, TW, ZI_DISPATCH_DTYPE(out_dt, TO, {
+            if (nv <= 2) ZI_LN_ROWS(2);
+            else if (nv <= 4) ZI_LN_ROWS(4);
+            else if (nv <= 6) ZI_LN_ROWS(6);
+            else if (nv <= 8) ZI_LN_ROWS(8);
+            else if (nv <= 12) ZI_LN_ROWS(12);
+            else if (nv <= 16) ZI_LN_ROWS(16);
+            else if (nv <= 24) ZI_LN_ROWS(24);
+            else ZI_LN_ROWS(32);
+        })));
+#undef ZI_LN_ROWS
+        return zi_check_launch("layer_norm");
+    }
+    if (aligned && splits <= 16 && hidden <= 8192) {
+        const int vecs = hidden / 4;
+        const int it = vecs > 1024 ? 2 : 1;
+        const int threads = ((vecs + it - 1) / it + ZI_WAVE - 1) / ZI_WAVE * ZI_WAVE;
+        ZI_DISPATCH_DTYPE(x_dt, TX, ZI_DISPATCH_DTYPE(w_dt, TW, ZI_DISPATCH_DTYPE(out_dt, TO, {
+            if (it == 1)
+                layer_norm_vec_kernel<TX, TW, TO, 1><<<n, threads, 0, stream>>>(
+                    (TO*)out, ldo, resid, (const TX*)x, splits, split_stride, ldx, (const TW*)w, (const TW*)b, hidden, eps);
+            else
+                layer_norm_vec_kernel<TX, TW, TO, 2><<<n, threads, 0, stream>>>(
+                    (TO*)out, ldo, resid, (const TX*)x, splits, split_stride, ldx, (const TW*)w, (const TW*)b, hidden, eps);
+        })));
+        return zi_check_launch("layer_norm");
+    }
     const bool wave_rows = n >= 64 && hidden <= LN_PER * ZI_WAVE;
     ZI_DISPATCH_DTYPE(x_dt, TX, ZI_DISPATCH_DTYPE(w_dt, TW, ZI_DISPATCH_DTYPE(out_dt, TO, {
         if (wave_rows)

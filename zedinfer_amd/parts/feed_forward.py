@@ -423,7 +423,13 @@ class ClampedExperts(FeedForward):
     def forward(self, x: torch.Tensor) -> torch.Tensor:
         n, E, top, ff, rt = x.shape[0], self.experts, self.top, self.ff, self.rt
         pairs = n * top
-        terms = rt.buffer("moe_terms", (2 if self.shared is not None else 1, n, self.hidden), torch.float32)
+        # the terms of the result: the routed experts' sum, then the shared expert's output (as the partial sums of
+        # its last product when that has few rows); whoever reads the stack adds them
+        shared_sums = 0
+        if self.shared is not None:
+            probe = rt.buffer("moe_shared_act", (n, self.shared.inter))
+            shared_sums = ops.linear_splits(n, self.hidden, self.shared.inter) if ops.linear_sums_supported(probe, self.shared.down) else 0
+        terms = rt.buffer("moe_terms", (1 + (shared_sums or (1 if self.shared is not None else 0)), n, self.hidden), torch.float32)
         z = ops.linear(x, self.router, out=rt.buffer("moe_logits", (n, E), torch.float32))
         idx = rt.buffer("moe_choice", (n, top), torch.int32)
         wt = rt.buffer("moe_weight", (n, top), torch.float32)
@@ -443,5 +449,8 @@ class ClampedExperts(FeedForward):
         ops.moe_combine(y, wt, place_of, terms[0])
         if self.shared is not None:
             act_s = self.shared.forward(rt, x, "moe_shared")
-            ops.linear(act_s, self.shared.down, out=terms[1])
+            if shared_sums:
+                ops.linear_sums(act_s, self.shared.down, out=terms[1:])
+            else:
+                ops.linear(act_s, self.shared.down, out=terms[1])
         return terms
