@@ -276,3 +276,32 @@ def test_activations_and_cap(dtype):
         ops.softcap(xd, 15.0)
         _close(xd, 15.0 * torch.tanh(x.double() / 15.0), 2e-6, "cap")
         assert float(xd.abs().max()) <= 15.0
+
+
+@pytest.mark.parametrize("T, n, nh, nkv, d, ps", [(300, 3, 4, 2, 64, 16), (1100, 8, 12, 2, 128, 16), (40, 16, 6, 6, 32, 8), (257, 1, 20, 4, 48, 8)])
+def test_the_projection_that_merges_the_chunks_counts_the_sink_once(T, n, nh, nkv, d, ps):
+    """Decoded tokens of n sequences (here: the same keys at n lengths): the attention kernel leaves the chunks of
+    keys unmerged, the output projection merges them; against the plain attention and a plain product."""
+    g = torch.Generator().manual_seed(T)
+    q, k, v = _attention_case(T, nh, nkv, d, ps, seed=T + 5, far=(T - 1, 2))
+    q, k, v = (x.to(torch.bfloat16) for x in (q, k, v))
+    sink = torch.tensor([2.0 - 0.9 * h for h in range(nh)], dtype=torch.float32)
+    w = (torch.randn(72, nh * d, generator=g) / (nh * d) ** 0.5).to(torch.bfloat16)
+    scale = 1.0 / math.sqrt(d)
+    att = plain.sink_attention(q.double(), k.double(), v.double(), scale, sink.double(), nh // nkv)
+    table, kc, vc = _fill_cache(k, v, ps, seed=T, dtype=torch.bfloat16)
+    # sequence i holds the first T - i tokens: its decoded token is the one at position T - 1 - i
+    pos = torch.tensor([T - 1 - i for i in range(n)], dtype=torch.int32, device=DEV)
+    qs = torch.stack([q[T - 1 - i].reshape(nh * d) for i in range(n)]).to(DEV)
+    tables = table.expand(n, -1).contiguous()
+    tok_seq = torch.arange(n, dtype=torch.int32, device=DEV)
+    assert ops.attention_decode_project_supported(w.to(DEV), n, nh, d)
+    ws = torch.empty(ops.attention_decode_workspace(n, nh, d), dtype=torch.float32, device=DEV)
+    assert ops.attention_decode(qs, kc, vc, tok_seq, pos, tables, nh, nkv, d, scale, T, workspace=ws, sinks=sink.to(DEV),
+                                leave_chunks=True) is None
+    sums = ops.attention_decode_project(ws, w.to(DEV), pos, nh, d, T, sinks=sink.to(DEV))
+    want = torch.stack([att[T - 1 - i].reshape(nh * d) for i in range(n)]) @ w.double().T
+    _close(sums.sum(0), want, 1.5e-2, "merged in the projection")
+    # without the sink the same call gives another result (the first heads' sinks are of the size of the scores)
+    other = ops.attention_decode_project(ws, w.to(DEV), pos, nh, d, T)
+    assert float((other.sum(0) - sums.sum(0)).abs().max()) > 1e-4

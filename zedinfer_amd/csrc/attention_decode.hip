@@ -592,7 +592,8 @@ template <int D>
 __global__ void __launch_bounds__(256)
 attention_decode_project_kernel(float* __restrict__ sums, const float* __restrict__ part_o,
                                 const float* __restrict__ part_ml, const int32_t* __restrict__ tok_pos, int n, int nh,
-                                int window, int max_chunks, const zi_bf16* __restrict__ w, int64_t ldw, int N, int hg) {
+                                int window, int max_chunks, const zi_bf16* __restrict__ w, int64_t ldw, int N, int hg,
+                                const float* __restrict__ sinks) {
     constexpr int DK = (D + 31) / 32;
     constexpr int XS = DK * 32 + 8;     // row stride of the merged head in LDS, in elements (16-byte rows, no bank repeat)
     __shared__ __attribute__((aligned(16))) uint16_t sx[16][XS];
@@ -671,6 +672,7 @@ attention_decode_project_kernel(float* __restrict__ sums, const float* __restric
                 }
             }
         }
+        if (sinks) L += __builtin_amdgcn_exp2f(sinks[h] * 1.4426950408889634f - M);      // the sink counts once
         {
             const float inv = count > max_chunks ? NAN : 1.f / L;      // chunks the launch did not cover: it shows
 #pragma unroll
@@ -810,7 +812,8 @@ extern "C" int zi_attention_decode_sink(void* out, const void* q, int dt, int n_
                                         int max_pages, int num_pages, int nh, int nkv, int d, int page_size, int window,
                                         float scale, int max_chunks, float* workspace, int64_t workspace_floats,
                                         const float* sinks, hipStream_t stream) {
-    ZI_REQUIRE(out != nullptr, "attention_decode_sink: the chunks cannot be left unmerged");
+    // out null: every token's chunks stay unmerged in the workspace for zi_attention_decode_project_sink, which
+    // counts the sink when it merges them
     return dec_launch("attention_decode_sink", out, q, dt, n_idx, ldq, ldo, kcache, vcache, tok_index, tok_seq, tok_pos,
                       block_tables, max_pages, num_pages, nh, nkv, d, page_size, window, scale, max_chunks, workspace,
                       workspace_floats, nullptr, sinks, stream);
@@ -877,9 +880,11 @@ extern "C" int zi_attention_decode_project_supported(int dt, int n, int nh, int 
 // max_chunks (and without tok_index): sums[s][t][:] = W[:, columns of the heads of group s] . attention
 // of token t, float32, s < ceil(nh / zi_attention_decode_project_heads(nh)), rows of `sums` N long.
 // W is [N, nh * d] bfloat16 with row stride ldw.
-extern "C" int zi_attention_decode_project(float* sums, const float* workspace, int64_t workspace_floats, int n,
-                                           const int32_t* tok_pos, int window, int max_chunks, const void* w, int dt,
-                                           int64_t ldw, int N, int nh, int d, hipStream_t stream) {
+// `sinks` (float32 [nh], or null): exp(sinks[h]) counts once in the denominator of head h's merge.
+extern "C" int zi_attention_decode_project_sink(float* sums, const float* workspace, int64_t workspace_floats, int n,
+                                                const int32_t* tok_pos, int window, int max_chunks, const void* w, int dt,
+                                                int64_t ldw, int N, int nh, int d, const float* sinks,
+                                                hipStream_t stream) {
     ZI_REQUIRE(zi_attention_decode_project_supported(dt, n, nh, d, ldw),
                "attention_decode_project: unsupported shape (bfloat16, 1..16 tokens, head_dim a multiple of 16 up to "
                "128, row stride a multiple of 8): dtype %d tokens %d heads %d head_dim %d stride %lld", dt, n, nh, d,
@@ -896,7 +901,7 @@ extern "C" int zi_attention_decode_project(float* sums, const float* workspace, 
     ZI_REQUIRE(grid.y <= 65535, "attention_decode_project: too many heads");
 #define ZI_DPJ(DD)                                                                                                    \
     attention_decode_project_kernel<DD><<<grid, 256, 0, stream>>>(sums, po, pml, tok_pos, n, nh, window, max_chunks,   \
-                                                                  (const zi_bf16*)w, ldw, N, hg)
+                                                                  (const zi_bf16*)w, ldw, N, hg, sinks)
     switch (d) {
         case 16: ZI_DPJ(16); break;
         case 32: ZI_DPJ(32); break;
@@ -909,4 +914,11 @@ extern "C" int zi_attention_decode_project(float* sums, const float* workspace, 
     }
 #undef ZI_DPJ
     return zi_check_launch("attention_decode_project");
+}
+
+extern "C" int zi_attention_decode_project(float* sums, const float* workspace, int64_t workspace_floats, int n,
+                                           const int32_t* tok_pos, int window, int max_chunks, const void* w, int dt,
+                                           int64_t ldw, int N, int nh, int d, hipStream_t stream) {
+    return zi_attention_decode_project_sink(sums, workspace, workspace_floats, n, tok_pos, window, max_chunks, w, dt, ldw, N,
+                                            nh, d, nullptr, stream);
 }

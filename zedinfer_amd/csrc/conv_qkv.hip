@@ -17,15 +17,22 @@
 #include "zi_api.h"
 
 #define CQ_THREADS 256
-#define CQ_MAX_CHANNELS 15360
+#define CQ_MAX_CHANNELS 15360      // with the angles (at most a head of them) within 64 KB of LDS
 #define CQ_MAX_TAPS 16
 
 // One value of the projection: the sum of its `splits` partial sums (split s at proj + s * split_stride), in rising order.
 template <typename TP>
 __device__ __forceinline__ float cq_value(const TP* __restrict__ proj, int64_t ld, int splits, int64_t split_stride,
                                           int64_t row, int c) {
-    float v = zi_load(proj + row * ld + c);
-    for (int s = 1; s < splits; ++s) v += zi_load(proj + s * split_stride + row * ld + c);
+    const TP* p = proj + row * ld + c;
+    float v = zi_load(p);
+    int s = 1;
+    for (; s + 4 <= splits; s += 4) {      // four loads in flight; the additions keep their order
+        const float a = zi_load(p + s * split_stride), b = zi_load(p + (s + 1) * split_stride),
+                    cc = zi_load(p + (s + 2) * split_stride), d = zi_load(p + (s + 3) * split_stride);
+        v += a; v += b; v += cc; v += d;
+    }
+    for (; s < splits; ++s) v += zi_load(p + s * split_stride);
     return v;
 }
 
@@ -81,17 +88,21 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
                 const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ entry_start,
                 const int32_t* __restrict__ entry_slot, const int32_t* __restrict__ slots, int64_t cache_slots, int nh,
                 int nkv, int dim, int vdim, int D, int taps, int page_size) {
-    extern __shared__ float y[];      // [C]
+    extern __shared__ float y[];      // [C] the convolved channels, q and k already times their gains; then [rot] angles
     __shared__ float red[16];
     const int t = blockIdx.x, e = tok_seq[t], local = t - entry_start[e];
     const int Qd = nh * dim, Kd = nkv * dim, Vd = nkv * vdim, C = Qd + Kd + Vd;
     float* tail = state + (int64_t)entry_slot[e] * state_stride;
     const int slot = slots ? slots[t] : -1;
     float sq = 0.f, sk = 0.f;
+    float* ang = y + C;      // (cos, sin) of the token's angles: the same for every head
+    if (table)
+        for (int i = threadIdx.x; i < rot; i += THREADS) ang[i] = table[(int64_t)t * rot + i];
     for (int c = threadIdx.x; c < C; c += THREADS) {
         float now;
+        const float gain = c < Qd ? q_norm[c] : (c < Qd + Kd ? k_norm[c - Qd] : 1.f);
         const float v = cq_conv<TP, TAPS>(proj, ld, splits, split_stride, bias, conv_w, tail, t, local, c, C, taps, now);
-        y[c] = v;
+        y[c] = v * gain;
         if (c < Qd) sq += v * v;
         else if (c < Qd + Kd) sk += v * v;
         // a step in which every entry brings one token: no other workgroup reads this entry's tail, and this thread
@@ -107,19 +118,17 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
     __syncthreads();
     const float rq = 1.f / sqrtf(sq / (float)Qd + eps), rk = 1.f / sqrtf(sk / (float)Kd + eps);
     const int half = rot / 2;
-    const float* ang = table ? table + (int64_t)t * half * 2 : nullptr;
     // queries: every (head, dim of the padded head)
     for (int i = threadIdx.x; i < nh * D; i += THREADS) {
         const int h = i / D, x = i % D;
         float v = 0.f;
         if (x < dim) {
             const int c = h * dim + x;
-            v = y[c] * rq * q_norm[c];
+            v = y[c] * rq;
             if (x < rot) {
                 const int p = x < half ? x : x - half;
                 const float cs = ang[2 * p], sn = ang[2 * p + 1];
-                const int co = x < half ? c + half : c - half;
-                const float o = y[co] * rq * q_norm[co];
+                const float o = y[x < half ? c + half : c - half] * rq;
                 v = x < half ? v * cs - o * sn : v * cs + o * sn;
             }
         }
@@ -132,12 +141,11 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
         float v = 0.f;
         if (x < dim) {
             const int c = g * dim + x;
-            v = y[Qd + c] * rk * k_norm[c];
+            v = y[Qd + c] * rk;
             if (x < rot) {
                 const int p = x < half ? x : x - half;
                 const float cs = ang[2 * p], sn = ang[2 * p + 1];
-                const int co = x < half ? c + half : c - half;
-                const float o = y[Qd + co] * rk * k_norm[co];
+                const float o = y[Qd + (x < half ? c + half : c - half)] * rk;
                 v = x < half ? v * cs - o * sn : v * cs + o * sn;
             }
         }
@@ -164,6 +172,7 @@ extern "C" int zi_conv_qkv(void* q_out, int dt, int64_t ldq, void* kcache, void*
                "conv_qkv: bad sizes (heads %d/%d, dim %d, vdim %d, head size %d, taps %d)", nh, nkv, dim, vdim, D, taps);
     const int64_t C = (int64_t)nh * dim + (int64_t)nkv * dim + (int64_t)nkv * vdim;
     ZI_REQUIRE(C <= CQ_MAX_CHANNELS, "conv_qkv: %lld channels are more than %d", (long long)C, CQ_MAX_CHANNELS);
+    ZI_REQUIRE((C + rot) * (int64_t)sizeof(float) <= 65000, "conv_qkv: channels and angles do not fit the workgroup's memory");
     ZI_REQUIRE(ld >= C && ldq >= (int64_t)nh * D, "conv_qkv: a row is too short");
     ZI_REQUIRE(state_stride >= (int64_t)(taps - 1) * C, "conv_qkv: the state row is too short");
     ZI_REQUIRE(rot >= 0 && rot % 2 == 0 && rot <= dim && (rot == 0 || table), "conv_qkv: %d rotated dims of %d", rot, dim);
@@ -172,7 +181,7 @@ extern "C" int zi_conv_qkv(void* q_out, int dt, int64_t ldq, void* kcache, void*
     ZI_REQUIRE(splits >= 1 && (splits == 1 || proj_dt == ZI_F32), "conv_qkv: partial sums are float32");
     ZI_REQUIRE(!move_tail || slots, "conv_qkv: moving the tail needs the tokens' slots");
     if (n == 0) return 0;
-    const size_t lds = (size_t)C * sizeof(float);
+    const size_t lds = (size_t)(C + rot) * sizeof(float);
     // few tokens: workgroups of 1,024 threads, so that a thread walks few channels one after the other
     const bool wide = n <= 512 && C > CQ_THREADS;
 #define ZI_CQ(TAPS, THREADS)                                                                                           \

@@ -163,6 +163,10 @@ int zi_attention_prefill_sink(void* out, const void* q, int dt, int num_tiles, i
     int32_t* entry_len, const int32_t* entry_past, const int32_t* block_tables, int max_pages, int num_pages, int nh,
     int nkv, int d, int page_size, int window, float scale, int rows, int max_chunks, float* workspace, int64_t
     workspace_floats, int tile, int alone, int chunk_keys, const float* sinks, hipStream_t stream);
+// attention_decode.hip
+int zi_attention_decode_project_sink(float* sums, const float* workspace, int64_t workspace_floats, int n, const int32_t*
+    tok_pos, int window, int max_chunks, const void* w, int dt, int64_t ldw, int N, int nh, int d, const float* sinks,
+    hipStream_t stream);
 // layer_norm.hip
 int zi_layer_norm(void* out, int out_dt, int64_t ldo, float* resid, const void* x, int x_dt, int splits, int64_t
     split_stride, int64_t ldx, const void* w, const void* b, int w_dt, int n, int hidden, float eps, hipStream_t
@@ -243,6 +247,7 @@ int zi_sample(int32_t* out, const float* logits, int64_t ld, float* work, int ro
     X(zi_attention_generic_sink) \
     X(zi_attention_decode_sink) \
     X(zi_attention_prefill_sink) \
+    X(zi_attention_decode_project_sink) \
     X(zi_layer_norm) \
     X(zi_conv_qkv) \
     X(zi_conv_tail) \

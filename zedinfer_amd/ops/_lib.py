@@ -89,6 +89,7 @@ _PROTOTYPES = {
     "zi_attention_decode_sink": [P, P, I, I, L, L, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, P, L, P, P],
     "zi_attention_prefill_sink": [P, P, I, I, L, L, P, P, P, P, P, P, P, P, I, I, I, I, I, I, I, F, I, I, P, L, I, I, I,
                                   P, P],
+    "zi_attention_decode_project_sink": [P, P, L, I, P, I, I, P, I, L, I, I, I, P, P],
     "zi_layer_norm": [P, I, L, P, P, I, I, L, L, P, P, I, I, I, F, P],
     "zi_conv_qkv": [P, I, L, P, P, P, I, L, I, L, P, P, P, L, I, P, P, F, P, I, I, P, P, P, P, L, I, I, I, I, I, I, I, P],
     "zi_conv_tail": [P, L, P, I, L, I, L, P, P, P, P, P, I, I, I, P],

@@ -415,23 +415,27 @@ def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
                      tok_pos: torch.Tensor, block_tables: torch.Tensor, nh: int, nkv: int, d: int, scale: float,
                      max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None,
                      tok_index: Optional[torch.Tensor] = None, workspace: Optional[torch.Tensor] = None,
-                     sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
+                     sinks: Optional[torch.Tensor] = None, leave_chunks: bool = False) -> Optional[torch.Tensor]:
     """The same attention for single query tokens, split over the keys, on the matrix cores
     (bfloat16, head_dim a multiple of 16 up to 128, group size <= 16, page size a multiple of 8).
     ``max_keys`` is an upper bound of the keys any listed token sees (its position + 1), known on
-    the host; it only sizes the launch."""
+    the host; it only sizes the launch.  ``leave_chunks`` (with ``sinks``, without a token list): nothing is merged
+    or written to ``out``; every token's chunks stay in ``workspace`` for ``attention_decode_project``."""
     out, n, count, ldq, ldo, pages, ps = _attention_args("attention_decode", q, kcache, vcache, tok_seq, tok_pos,
-                                                         block_tables, nh, nkv, d, tok_index, out)
+                                                         block_tables, nh, nkv, d, tok_index,
+                                                         q if (leave_chunks and out is None) else out)   # (nothing is written there)
+    if leave_chunks and (sinks is None or tok_index is not None or workspace is None):
+        raise ValueError("attention_decode: chunks are left for mixers with sinks, all tokens, in a given workspace")
     if window > 0:
         max_keys = min(max_keys, window)
     max_chunks = int(_lib.load().zi_attention_decode_chunks(int(max_keys)))
     need = attention_decode_workspace(count, nh, d)
-    if max_chunks > 1:
+    if max_chunks > 1 or leave_chunks:
         if workspace is None:
             workspace = torch.empty((need,), dtype=torch.float32, device=q.device)
         if workspace.dtype != torch.float32 or workspace.numel() < need or not workspace.is_contiguous():
             raise ValueError(f"attention_decode: workspace must be a contiguous float32 buffer of {need} entries")
-    args = (_p(out), _p(q), _code(q, "attention_decode"), count, ldq, ldo, _p(kcache),
+    args = (_p(None if leave_chunks else out), _p(q), _code(q, "attention_decode"), count, ldq, ldo, _p(kcache),
             _p(vcache), _p(tok_index), _p(tok_seq), _p(tok_pos), _p(block_tables), block_tables.shape[1], pages,
             nh, nkv, d, ps, int(window), float(scale), max_chunks, _p(workspace),
             workspace.numel() if workspace is not None else 0)
@@ -439,7 +443,7 @@ def attention_decode(q: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor
         _lib.call("zi_attention_decode_sink", *args, _p(_sinks(sinks, nh, q, "attention_decode")), _stream())
     else:
         _lib.call("zi_attention_decode", *args, _stream())
-    return out
+    return None if leave_chunks else out
 
 
 def rope_table(pos: torch.Tensor, inv_freq: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -552,7 +556,8 @@ def attention_decode_project_splits(nh: int) -> int:
 
 
 def attention_decode_project(workspace: torch.Tensor, weight: torch.Tensor, tok_pos: torch.Tensor, nh: int, d: int,
-                             max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                             max_keys: int, window: int = 0, out: Optional[torch.Tensor] = None,
+                             sinks: Optional[torch.Tensor] = None) -> torch.Tensor:
     """The output projection of decoded tokens straight from the chunks that ``attention_decode_fused(...,
     leave_chunks=True)`` left in ``workspace`` (same tokens, heads, ``max_keys`` and ``window``): float32
     partial sums [splits, n, N] over groups of heads, to be added in rising order.  ``weight`` is [N, nh*d]."""
@@ -574,8 +579,12 @@ def attention_decode_project(workspace: torch.Tensor, weight: torch.Tensor, tok_
     if window > 0:
         max_keys = min(max_keys, window)
     max_chunks = int(_lib.load().zi_attention_decode_chunks(int(max_keys)))
-    _lib.call("zi_attention_decode_project", _p(out), _p(workspace), workspace.numel(), n, _p(tok_pos), int(window),
-              max_chunks, _p(weight), _code(weight, "attention_decode_project"), weight.stride(0), N, nh, d, _stream())
+    args = (_p(out), _p(workspace), workspace.numel(), n, _p(tok_pos), int(window), max_chunks, _p(weight),
+            _code(weight, "attention_decode_project"), weight.stride(0), N, nh, d)
+    if sinks is not None:      # (float32 [nh]: exp(sinks[h]) counts once in the denominator of head h's merge)
+        _lib.call("zi_attention_decode_project_sink", *args, _p(_sinks(sinks, nh, weight, "attention_decode_project")), _stream())
+    else:
+        _lib.call("zi_attention_decode_project", *args, _stream())
     return out
 
 

@@ -500,6 +500,27 @@ class ConvAttention(Attention):
         if not single:
             ops.conv_tail(memory.state, proj, self.bias, batch.entry_start, batch.entry_len, batch.entry_slot, self.taps,
                           slots=view.slots)
+        out = self.decode_and_project(q, batch, view, memory) if single else None
+        if out is not None:
+            return out
         att = rt.buffer("attn_out", (n, self.qd))
         self.attend(q, att, batch, view, memory)
         return self.project(att, n)
+
+    def decode_and_project(self, q, batch, view, memory: LayerMemory) -> Optional[torch.Tensor]:
+        """A pure decode step of few tokens: the attention kernel leaves every token's chunks of keys unmerged and
+        the output projection merges them (and counts the sink) as it loads its operand: one launch less a layer,
+        as the first architecture's decode steps do.  None: the shape is not taken, nothing was done."""
+        n = q.shape[0]
+        kc, vc = memory.tensors["k"], memory.tensors["v"]
+        if (n > self.FUSED_DECODE_MAX_TOKENS or self.o.numel() * self.o.element_size() > self.PROJECT_FROM_CHUNKS_MAX_BYTES
+                or not ops.attention_decode_supported(q.dtype, self.nh, self.nkv, self.d, kc.shape[2])
+                or not ops.attention_decode_project_supported(self.o, n, self.nh, self.d)):
+            return None
+        max_keys = batch.plans[self.plan_key].sizes["max_short_keys"]
+        ws = self.rt.buffer("attn_split", (ops.attention_decode_workspace(n, self.nh, self.d),), torch.float32)
+        ops.attention_decode(q, kc, vc, batch.tok_seq, batch.positions, view.block_tables, self.nh, self.nkv, self.d,
+                             self.scale, max_keys, self.window, workspace=ws, sinks=self.sinks, leave_chunks=True)
+        out = self.rt.buffer("attn_proj_heads", (ops.attention_decode_project_splits(self.nh), n, self.hidden), torch.float32)
+        return ops.attention_decode_project(ws, self.o, batch.positions, self.nh, self.d, max_keys, self.window, out=out,
+                                            sinks=self.sinks)
