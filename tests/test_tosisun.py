@@ -52,6 +52,20 @@ def test_a_layer_with_anothers_weights_is_that_layers_parts_on_a_cache_of_its_ow
     assert tosisun_forward_config(TosisunConfig.from_dict(models.ODD)).lm_head.params["softcap"] is None
 
 
+def test_weights_of_may_lead_over_another_such_layer_and_to_a_later_one():
+    cfg = copy.deepcopy(models.MAIN)
+    cfg["layers"][4]["weights_of"] = 0
+    cfg["layers"].append(copy.deepcopy(cfg["layers"][2]))      # layer 6 -> 2 -> 1
+    cfg["layers"][6]["weights_of"] = 2
+    cfg["layers"][0], cfg["layers"][4] = cfg["layers"][4], cfg["layers"][0]      # layer 0 now runs with layer 4's tensors
+    cfg["layers"][0]["weights_of"] = 4
+    c = TosisunConfig.from_dict(cfg)
+    assert [c.owner_of(i) for i in range(7)] == [4, 1, 1, 3, 4, 5, 1]
+    fc = tosisun_forward_config(c)
+    assert [(s.layer, s.cache) for s in fc.schedule] == [(2, 0), (0, 1), (0, 2), (1, 3), (2, 4), (3, 5), (0, 6)]
+    assert "l4.mix.q" in expected_weights(fc) and "l0.mix.q" not in expected_weights(fc)
+
+
 def _broken(change):
     cfg = copy.deepcopy(models.MAIN)
     change(cfg)
@@ -68,7 +82,8 @@ def _broken(change):
     (lambda c: c["layers"][0]["mixer"]["rot"].update(dims=40), "rot"),
     (lambda c: c["layers"][0]["mixer"]["rot"]["scaling"].pop("high"), "scaling"),
     (lambda c: c["layers"][2].update(weights_of=2), "weights_of"),
-    (lambda c: c["layers"][4].update(weights_of=2), "weights_of"),
+    (lambda c: c["layers"][4].update(weights_of=9), "weights_of"),
+    (lambda c: (c["layers"][1].update(weights_of=2), c["layers"][2].update(weights_of=1)), "weights_of"),
     (lambda c: c["layers"][2]["mixer"].update(dim=32), "weights"),
     (lambda c: c["layers"][1]["mlp"]["router"].update(top=7), "top"),
     (lambda c: c["layers"][1]["mlp"]["expert"].pop("limit"), "limit"),

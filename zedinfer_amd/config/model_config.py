@@ -328,12 +328,8 @@ class TosisunConfig(ModelConfig):
             kind = layer.get("type") if isinstance(layer, Mapping) else None
             if kind not in self.MIXER_KEYS:
                 raise ConfigError(f"config.json: layer {i} has type {kind!r}; known: {', '.join(sorted(self.MIXER_KEYS))}")
-            src = layer.get("weights_of")
-            if src is not None:
-                ok = isinstance(src, int) and not isinstance(src, bool) and 0 <= src < i \
-                    and self.layers[src].get("weights_of") is None
-                if not ok:
-                    raise ConfigError(f"config.json: layer {i}: weights_of must name an earlier layer with tensors of its own")
+            if layer.get("weights_of") is not None:
+                src = self.owner_of(i)
                 o = self.layers[src]
                 if (o.get("type"), o.get("mixer"), o.get("mlp")) != (layer.get("type"), layer.get("mixer"), layer.get("mlp")):
                     raise ConfigError(f"config.json: layer {i}: a layer that uses layer {src}'s weights must equal it in "
@@ -371,6 +367,19 @@ class TosisunConfig(ModelConfig):
                     raise ConfigError(f"config.json: layer {i}: a shared expert needs ff and limit")
             else:
                 raise ConfigError(f"config.json: layer {i}: mlp.kind {mlp.get('kind')!r} is neither 'dense' nor 'moe'")
+
+    def owner_of(self, i: int) -> int:
+        """The layer whose tensors layer ``i`` runs with: itself, or what its ``weights_of`` names (followed to a
+        layer that has tensors of its own; it may stand before or after)."""
+        seen = set()
+        while isinstance(self.layers[i], Mapping) and self.layers[i].get("weights_of") is not None:
+            src = self.layers[i]["weights_of"]
+            if isinstance(src, bool) or not isinstance(src, int) or not (0 <= src < len(self.layers)) or src == i or src in seen:
+                raise ConfigError(f"config.json: layer {i}: weights_of must name another layer of the model, and lead to one "
+                                  "with tensors of its own")
+            seen.add(i)
+            i = src
+        return i
 
     def to_dict(self) -> Dict[str, Any]:
         d = {"architecture": self.architectures[0] if self.architectures else "Tosisun",

@@ -71,13 +71,13 @@ def tosisun_forward_config(cfg: TosisunConfig) -> ModelForwardConfig:
     H = cfg.hidden_size
     layers, schedule, built = [], [], {}
     for i, layer in enumerate(cfg.layers):
-        src = layer.get("weights_of")
-        if src is None:
+        if layer.get("weights_of") is None:
             built[i] = len(layers)
             layers.append(LayerSpec("output_norm", _mixer(cfg, i), _feed_forward(cfg, i),
                                     {"mixer_out": _norm(cfg, f"l{i}.norm1"), "ff_out": _norm(cfg, f"l{i}.norm2")}))
+    for i in range(len(cfg.layers)):
         # a layer that runs with another's tensors is that layer's parts once more, on a cache and state of its own
-        schedule.append(ScheduleStep(layer=built[i if src is None else int(src)], cache=i))
+        schedule.append(ScheduleStep(layer=built[cfg.owner_of(i)], cache=i))
     fc = ModelForwardConfig(
         architecture="Tosisun", hidden_size=H, vocab_size=cfg.vocab_size,
         embedding=PartSpec("token", {"vocab_size": cfg.vocab_size, "hidden_size": H}, {"weight": "embed"}),
