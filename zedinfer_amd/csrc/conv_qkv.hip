@@ -36,46 +36,60 @@ __device__ __forceinline__ float cq_value(const TP* __restrict__ proj, int64_t l
     return v;
 }
 
-// The convolved value of channel c of token t; `now` receives the token's own input (projection + bias).  With the
-// number of taps known at compile time (TAPS > 0) and float32 rows that are no partial sums, every tap's input is one
-// load whose address alone depends on where it comes from (the projection or the tail), so all are in flight together.
+// The convolved value of channel c of token t.  With the number of taps known at compile time (TAPS > 0) the taps'
+// inputs (projection + bias, or the tail's rows) come back in `u`, the token's own last, so that the kernel can move
+// the tail on without reading it again; with float32 rows that are no partial sums every input is one load whose
+// address alone depends on where it comes from, so all are in flight together.  TAPS == 0: any number of taps, and
+// `u[0]` is the token's own input.
 template <typename TP, int TAPS>
 __device__ __forceinline__ float cq_conv(const TP* __restrict__ proj, int64_t ld, int splits, int64_t split_stride,
                                          const float* __restrict__ bias, const float* __restrict__ conv_w,
                                          const float* __restrict__ tail, int t, int local, int c, int C, int taps,
-                                         float& now) {
+                                         float* u) {
     const float bc = bias ? bias[c] : 0.f;
-    if constexpr (TAPS > 0 && sizeof(TP) == 4) {
-        if (splits == 1) {
-            float u[TAPS], wv[TAPS];
+    if constexpr (TAPS > 0) {
+        float wv[TAPS];
 #pragma unroll
-            for (int j = 0; j < TAPS; ++j) {
-                const int li = local - (TAPS - 1) + j;
-                const float* src = li >= 0 ? (const float*)proj + (int64_t)(t - local + li) * ld + c
-                                           : tail + (int64_t)(li + TAPS - 1) * C + c;
-                u[j] = *src;
-                wv[j] = conv_w[(int64_t)c * TAPS + j];
-            }
-            float y = 0.f;
+        for (int j = 0; j < TAPS; ++j) wv[j] = conv_w[(int64_t)c * TAPS + j];
+        bool done = false;
+        if constexpr (sizeof(TP) == 4) {
+            if (splits == 1) {
 #pragma unroll
-            for (int j = 0; j < TAPS; ++j) {
-                const int li = local - (TAPS - 1) + j;
-                if (li >= 0) u[j] += bc;
-                y += wv[j] * u[j];
+                for (int j = 0; j < TAPS; ++j) {
+                    const int li = local - (TAPS - 1) + j;
+                    const float* src = li >= 0 ? (const float*)proj + (int64_t)(t - local + li) * ld + c
+                                               : tail + (int64_t)(li + TAPS - 1) * C + c;
+                    u[j] = *src;
+                }
+#pragma unroll
+                for (int j = 0; j < TAPS; ++j)
+                    if (local - (TAPS - 1) + j >= 0) u[j] += bc;
+                done = true;
             }
-            now = u[TAPS - 1];
-            return y;
         }
+        if (!done) {
+#pragma unroll
+            for (int j = 0; j < TAPS; ++j) {
+                const int li = local - (TAPS - 1) + j;
+                u[j] = li >= 0 ? cq_value(proj, ld, splits, split_stride, t - local + li, c) + bc
+                               : tail[(int64_t)(li + TAPS - 1) * C + c];
+            }
+        }
+        float y = 0.f;
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) y += wv[j] * u[j];
+        return y;
+    } else {
+        u[0] = cq_value(proj, ld, splits, split_stride, t, c) + bc;
+        float y = conv_w[(int64_t)c * taps + taps - 1] * u[0];
+        for (int j = 0; j + 1 < taps; ++j) {
+            const int li = local - (taps - 1) + j;
+            const float x = li >= 0 ? cq_value(proj, ld, splits, split_stride, t - local + li, c) + bc
+                                    : tail[(int64_t)(li + taps - 1) * C + c];
+            y += conv_w[(int64_t)c * taps + j] * x;
+        }
+        return y;
     }
-    now = cq_value(proj, ld, splits, split_stride, t, c) + bc;
-    float y = conv_w[(int64_t)c * taps + taps - 1] * now;
-    for (int j = 0; j + 1 < taps; ++j) {
-        const int li = local - (taps - 1) + j;
-        const float u = li >= 0 ? cq_value(proj, ld, splits, split_stride, t - local + li, c) + bc
-                                : tail[(int64_t)(li + taps - 1) * C + c];
-        y += conv_w[(int64_t)c * taps + j] * u;
-    }
-    return y;
 }
 
 template <typename TP, typename T, int TAPS, int THREADS>
@@ -99,9 +113,9 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
     if (table)
         for (int i = threadIdx.x; i < rot; i += THREADS) ang[i] = table[(int64_t)t * rot + i];
     for (int c = threadIdx.x; c < C; c += THREADS) {
-        float now;
+        float u[TAPS > 0 ? TAPS : 1];
         const float gain = c < Qd ? q_norm[c] : (c < Qd + Kd ? k_norm[c - Qd] : 1.f);
-        const float v = cq_conv<TP, TAPS>(proj, ld, splits, split_stride, bias, conv_w, tail, t, local, c, C, taps, now);
+        const float v = cq_conv<TP, TAPS>(proj, ld, splits, split_stride, bias, conv_w, tail, t, local, c, C, taps, u);
         y[c] = v * gain;
         if (c < Qd) sq += v * v;
         else if (c < Qd + Kd) sk += v * v;
@@ -109,8 +123,13 @@ conv_qkv_kernel(T* __restrict__ q_out, int64_t ldq, T* __restrict__ kcache, T* _
         // alone reads and writes channel c of it, so the tail moves on here (a token without a place in the cache is
         // padding and moves nothing)
         if (move_tail && slot >= 0 && taps > 1) {
-            for (int k = 0; k + 2 < taps; ++k) tail[(int64_t)k * C + c] = tail[(int64_t)(k + 1) * C + c];
-            tail[(int64_t)(taps - 2) * C + c] = now;
+            if constexpr (TAPS > 0) {
+#pragma unroll
+                for (int k = 0; k + 1 < TAPS; ++k) tail[(int64_t)k * C + c] = u[k + 1];
+            } else {
+                for (int k = 0; k + 2 < taps; ++k) tail[(int64_t)k * C + c] = tail[(int64_t)(k + 1) * C + c];
+                tail[(int64_t)(taps - 2) * C + c] = u[0];
+            }
         }
     }
     sq = zi_block_sum(sq, red);
