@@ -126,7 +126,7 @@ def test_in_float32_every_cut_gives_the_same_bits(tmp_path):
     prompts, of portions and of a mixed batch agree to the last bit."""
     name = "main"
     vocab = models.CONFIGS[name]["vocab"]
-    requests = {f"b{i}": traces.random_tokens(vocab, n, seed=140 + i) for i, n in enumerate([33, 50, 6])}
+    requests = {f"b{i}": traces.random_tokens(vocab, n, seed=140 + i) for i, n in enumerate([33, 150, 6])}
     folder, cfg, w, engine = _setup(tmp_path, name, "float32", pages=64)
     rows = {}
     for what, steps in (("whole", traces.whole(requests)), ("portions", traces.portions(requests, seed=3, sizes=(2, 5, 1, 7))),
@@ -141,7 +141,7 @@ def test_in_float32_every_cut_gives_the_same_bits(tmp_path):
                     rows.setdefault((e["id"], base + wpos), []).append(out[st["step"]][row].copy())
                     row += 1
                 fed[e["id"]] = base + len(e["tokens"])
-    assert len(rows) == 33 + 50 + 6
+    assert len(rows) == 33 + 150 + 6
     for key, got in rows.items():
         assert len(got) == 3 and np.array_equal(got[0], got[1]) and np.array_equal(got[0], got[2]), key
 

@@ -201,8 +201,10 @@ extern "C" int zi_conv_qkv(void* q_out, int dt, int64_t ldq, void* kcache, void*
     ZI_REQUIRE(!move_tail || slots, "conv_qkv: moving the tail needs the tokens' slots");
     if (n == 0) return 0;
     const size_t lds = (size_t)(C + rot) * sizeof(float);
-    // few tokens: workgroups of 1,024 threads, so that a thread walks few channels one after the other
-    const bool wide = n <= 512 && C > CQ_THREADS;
+    // few tokens: workgroups of 1,024 threads, so that a thread walks few channels one after the other (with bfloat16
+    // results only: the two sizes add the squares in different orders, and the float32 path keeps one order whatever
+    // the step holds)
+    const bool wide = n <= 512 && C > CQ_THREADS && dt == ZI_BF16;
 #define ZI_CQ(TAPS, THREADS)                                                                                           \
     conv_qkv_kernel<TP, T, TAPS, THREADS><<<n, THREADS, lds, stream>>>(                                                \
         (T*)q_out, ldq, (T*)kcache, (T*)vcache, (const TP*)proj, ld, splits, split_stride, bias, conv_w, state,       \

@@ -9,8 +9,8 @@
 // receives y.
 //
 // One workgroup per row; a thread keeps its values of the row in registers (up to LN_PER * LN_THREADS columns),
-// wider rows are read again from memory.  From 64 rows on and rows of at most 64 * LN_PER columns a wavefront takes
-// a row and no barrier is needed.  Sums run in an order fixed by the row's width alone.
+// wider rows are read again from memory.  Rows of at most 64 * LN_PER columns are taken by a wavefront each and no
+// barrier is needed.  Sums run in an order fixed by the row's width alone.
 #include "zi_common.h"
 #include "zi_api.h"
 
@@ -160,7 +160,7 @@ __global__ void layer_norm_vec_kernel(TO* __restrict__ out, int64_t ldo, float* 
     }
 }
 
-// Many rows, one or two terms: a wavefront per row, four rows a workgroup, no barrier.  A lane owns NV groups of four
+// One or two terms: a wavefront per row, four rows a workgroup, no barrier.  A lane owns NV groups of four
 // consecutive values, 256 values apart (every load instruction of the wavefront reads 1 KB of the row).
 template <typename TX, typename TW, typename TO, int NV>
 __global__ void __launch_bounds__(4 * ZI_WAVE)
@@ -226,7 +226,9 @@ extern "C" int zi_layer_norm(void* out, int out_dt, int64_t ldo, float* resid, c
                          ((uintptr_t)w % 16) == 0 && ((uintptr_t)b % 16) == 0 && ((uintptr_t)resid % 16) == 0 &&
                          ((uintptr_t)out % 16) == 0 && ldo % 4 == 0 && (x_dt == ZI_F32 || (ldx % 8 == 0 && ((uintptr_t)x % 8) == 0)) &&
                          !(x_dt == ZI_BF16 && splits > 1);
-    if (aligned && n >= 64 && splits <= 2 && hidden <= 8192) {
+    // Which kernel runs depends on the row's width and the number of terms, never on the number of rows: a row's sums
+    // are then the same whatever else is in the step.
+    if (aligned && splits <= 2 && hidden <= 8192) {
         const int nv = (hidden + 4 * ZI_WAVE - 1) / (4 * ZI_WAVE);
         const int wgs = (n + 3) / 4;
 #define ZI_LN_ROWS(NV)                                                                                                \
@@ -259,7 +261,7 @@ extern "C" int zi_layer_norm(void* out, int out_dt, int64_t ldo, float* resid, c
         })));
         return zi_check_launch("layer_norm");
     }
-    const bool wave_rows = n >= 64 && hidden <= LN_PER * ZI_WAVE;
+    const bool wave_rows = hidden <= LN_PER * ZI_WAVE;
     ZI_DISPATCH_DTYPE(x_dt, TX, ZI_DISPATCH_DTYPE(w_dt, TW, ZI_DISPATCH_DTYPE(out_dt, TO, {
         if (wave_rows)
             layer_norm_kernel<TX, TW, TO, ZI_WAVE><<<(n + 3) / 4, LN_THREADS, 0, stream>>>(
