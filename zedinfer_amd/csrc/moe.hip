@@ -211,6 +211,16 @@ extern "C" int zi_moe_group(int32_t* plan, int32_t* order, int32_t* place_of, co
 #define MOE_ACT_NONE 0
 #define MOE_ACT_GELU_ERF 1
 
+__device__ __forceinline__ void moe_store4(float* p, float a, float b, float c, float d) {
+    *reinterpret_cast<float4*>(p) = make_float4(a, b, c, d);
+}
+__device__ __forceinline__ void moe_store4(zi_bf16* p, float a, float b, float c, float d) {
+    uint2 v;
+    v.x = zi_pack_bf16x2(a, b);
+    v.y = zi_pack_bf16x2(c, d);
+    *reinterpret_cast<uint2*>(p) = v;
+}
+
 __device__ __forceinline__ float moe_act(float z, int act) {
     return act == MOE_ACT_GELU_ERF ? 0.5f * z * (1.f + erff(z * 0.70710678118654752440f)) : z;
 }
@@ -322,17 +332,26 @@ moe_linear_mfma_kernel(TO* __restrict__ out, int64_t ldo, const zi_bf16* __restr
             for (int c = 0; c < CT; ++c)
                 acc[t][c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[c].b, b[t].b, acc[t][c], 0, 0, 0);
     }
+    // a lane holds four consecutive columns of a row: one store of 16 (float32) or 8 bytes (bfloat16) where the rows
+    // allow it
+    const bool whole = ldo % 4 == 0 && ((uintptr_t)out % 16) == 0;
 #pragma unroll
     for (int t = 0; t < RT; ++t) {
         const int row = t * 16 + r;
         if (row >= rows) continue;
 #pragma unroll
-        for (int c = 0; c < CT; ++c)
+        for (int c = 0; c < CT; ++c) {
+            const int n = n0 + 16 * c + 4 * j;
+            TO* dst = out + (int64_t)(r0 + row) * ldo + n;
+            if (whole && n + 3 < N) {
+                moe_store4(dst, moe_act(acc[t][c][0], act), moe_act(acc[t][c][1], act), moe_act(acc[t][c][2], act),
+                           moe_act(acc[t][c][3], act));
+            } else {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                const int n = n0 + 16 * c + 4 * j + i;
-                if (n < N) zi_store(out + (int64_t)(r0 + row) * ldo + n, moe_act(acc[t][c][i], act));
+                for (int i = 0; i < 4; ++i)
+                    if (n + i < N) zi_store(dst + i, moe_act(acc[t][c][i], act));
             }
+        }
     }
 }
 

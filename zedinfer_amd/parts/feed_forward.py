@@ -441,9 +441,7 @@ class ClampedExperts(FeedForward):
         order = rt.buffer("moe_order", (pairs,), torch.int32)
         place_of = rt.buffer("moe_place", (pairs,), torch.int32)
         ops.moe_group(idx, E, rows, plan, order, place_of)
-        # the gate/up results: float32 for few tokens, the activation type for many (half the traffic of what is the
-        # largest array of a prompt step)
-        gu = rt.buffer("moe_gate_up", (pairs, 2 * ff), torch.float32 if n <= ops.FEW_ROWS else rt.dtype)
+        gu = rt.buffer("moe_gate_up", (pairs, 2 * ff), torch.float32)
         ops.moe_linear(x, self.gate_up, plan, rows, tiles, out=gu, source=order, source_div=top)
         act = rt.buffer("moe_act", (pairs, ff))
         ops.clamped_glu(gu[:, :ff], gu[:, ff:], self.limit, out=act)
