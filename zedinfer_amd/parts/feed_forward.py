@@ -356,8 +356,7 @@ class _ClampedGated:
             gu = ops.linear_sums(x, self.gate_up, out=rt.buffer(name + "_gate_up_sums", (S, n, self.up_at + I), torch.float32))
             ops.clamped_glu(gu[:, :, :I], gu[:, :, self.up_at:], self.limit, out=act)
         else:
-            gu = ops.linear(x, self.gate_up, out=rt.buffer(name + "_gate_up", (n, self.up_at + I),
-                                                           torch.float32 if n <= ops.FEW_ROWS else rt.dtype))
+            gu = ops.linear(x, self.gate_up, out=rt.buffer(name + "_gate_up", (n, self.up_at + I), torch.float32))
             ops.clamped_glu(gu[:, :I], gu[:, self.up_at:], self.limit, out=act)
         return act
 
