@@ -417,7 +417,7 @@ def tosisun_shape(size, layers, vocab):
     out = []
     for i in range(layers):
         mixer = dict(heads=z["heads"], kv_heads=max(2, z["heads"] // 7), dim=128, vdim=128, conv=4, scale=128 ** -0.5,
-                     rot=dict(base=500000.0, dims=64, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
+                     rot=dict(base=1000000.0, dims=64, scaling=dict(factor=8.0, low=1.0, high=4.0, original=8192)))
         mlp = dict(kind="dense", ff=z["ff"]) if i % 2 == 0 else \
             dict(kind="moe", expert=dict(ff=z["expert_ff"], limit=7.0), router=dict(experts=z["experts"], top=z["top"]),
                  shared=dict(ff=z["expert_ff"], limit=7.0))

@@ -145,8 +145,8 @@ def test_the_frequencies_of_the_part_are_the_plain_ones_and_all_three_branches_o
     s = (64 / wl - 1.0) / 3.0
     assert abs(f[1] - ((1 - s) * plainf[1] / 8.0 + s * plainf[1])) < 1e-15
     np.testing.assert_allclose(stretched_frequencies(8, 10000.0, sc), np.array(f, dtype=np.float32), rtol=1e-7)
-    np.testing.assert_allclose(stretched_frequencies(32, 500000.0, dict(factor=4.0, low=1.0, high=4.0, original=32)),
-                               np.array(plain.stretched_frequencies(32, 500000.0, dict(factor=4.0, low=1.0, high=4.0, original=32)),
+    np.testing.assert_allclose(stretched_frequencies(32, 1000000.0, dict(factor=4.0, low=1.0, high=4.0, original=32)),
+                               np.array(plain.stretched_frequencies(32, 1000000.0, dict(factor=4.0, low=1.0, high=4.0, original=32)),
                                         dtype=np.float32), rtol=1e-7)
     assert plain.stretched_frequencies(6, 100.0, None) == [100.0 ** (-2.0 * i / 6) for i in range(3)]
 

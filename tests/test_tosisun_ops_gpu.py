@@ -273,9 +273,9 @@ def test_activations_and_cap(dtype):
         _close(o2, torch.clamp(parts.double().sum(0), min=0) ** 2, 3e-6, "relu squared of sums")
         x = 40 * torch.randn(n, I, generator=g)
         xd = x.to(DEV)
-        ops.softcap(xd, 15.0)
-        _close(xd, 15.0 * torch.tanh(x.double() / 15.0), 2e-6, "cap")
-        assert float(xd.abs().max()) <= 15.0
+        ops.softcap(xd, 12.0)
+        _close(xd, 12.0 * torch.tanh(x.double() / 12.0), 2e-6, "cap")
+        assert float(xd.abs().max()) <= 12.0
 
 
 @pytest.mark.parametrize("T, n, nh, nkv, d, ps", [(300, 3, 4, 2, 64, 16), (1100, 8, 12, 2, 128, 16), (40, 16, 6, 6, 32, 8), (257, 1, 20, 4, 48, 8)])
@@ -305,3 +305,66 @@ def test_the_projection_that_merges_the_chunks_counts_the_sink_once(T, n, nh, nk
     # without the sink the same call gives another result (the first heads' sinks are of the size of the scores)
     other = ops.attention_decode_project(ws, w.to(DEV), pos, nh, d, T)
     assert float((other.sum(0) - sums.sum(0)).abs().max()) > 1e-4
+
+
+# ---- the feed-forwards as parts --------------------------------------------------------------------------------------
+def _part(registry, kind, params, weights, dtype):
+    from zedinfer_amd.config.forward_config import PartSpec
+    from zedinfer_amd.parts import Runtime
+    rt = Runtime(DEV, dtype)
+    spec = PartSpec(kind, params, {k: k for k in weights})
+    return registry.get(kind)(spec, {k: v.to(DEV, dtype) for k, v in weights.items()}, rt)
+
+
+def _sum_terms(y):
+    return (y.sum(0) if y.dim() == 3 else y).double().cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n, H, I", [(1, 64, 40), (9, 96, 136), (70, 72, 52), (200, 128, 256)])
+def test_the_relu_squared_feed_forward(n, H, I, dtype):
+    from zedinfer_amd.parts import FEED_FORWARDS
+    g = torch.Generator().manual_seed(n + I)
+    w = {"up": torch.randn(I, H, generator=g) / H ** 0.5, "down": torch.randn(H, I, generator=g) / I ** 0.5}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    x = torch.randn(n, H, generator=g).to(dtype)
+    ff = _part(FEED_FORWARDS, "relu2_mlp", {"hidden_size": H, "intermediate_size": I}, w, dtype)
+    got = _sum_terms(ff.forward(x.to(DEV)))
+    want = plain.relu_squared_mlp(x.double(), w["up"].double(), w["down"].double())
+    _close(got, want, 1e-5 if dtype == torch.float32 else 2e-2, "relu squared mlp")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("n, H, E, top, ff, sff", [(1, 64, 4, 2, 24, 16), (13, 96, 6, 3, 40, 56), (90, 72, 5, 1, 36, 0),
+                                                 (300, 128, 16, 4, 64, 96), (7, 48, 3, 3, 20, 12)])
+def test_the_clamped_experts(n, H, E, top, ff, sff, dtype):
+    """Router with bias, the choice of the largest logits, clamped experts, the shared expert: against the plain
+    feed-forward.  The tokens' router logits are spread so that no choice is a close call under rounding."""
+    from zedinfer_amd.parts import FEED_FORWARDS
+    g = torch.Generator().manual_seed(n + E)
+    w = {"router": 3.0 * torch.randn(E, H, generator=g) / H ** 0.5, "router_bias": 0.5 * torch.randn(E, generator=g)}
+    for e in range(E):
+        w.update({f"gate_{e}": 2 * torch.randn(ff, H, generator=g) / H ** 0.5, f"up_{e}": 2 * torch.randn(ff, H, generator=g) / H ** 0.5,
+                  f"down_{e}": torch.randn(H, ff, generator=g) / ff ** 0.5})
+    if sff:
+        w.update({"shared_gate": 2 * torch.randn(sff, H, generator=g) / H ** 0.5, "shared_up": 2 * torch.randn(sff, H, generator=g) / H ** 0.5,
+                  "shared_down": torch.randn(H, sff, generator=g) / sff ** 0.5})
+    w = {k: v.to(dtype) for k, v in w.items()}
+    x = torch.randn(4 * n, H, generator=g).to(dtype)
+    z = x.double() @ w["router"].double().T + w["router_bias"].double()
+    zs = torch.sort(z, dim=1, descending=True).values
+    clear = torch.ones(4 * n, dtype=torch.bool) if top == E else (zs[:, top - 1] - zs[:, top]) > 0.1
+    x = x[clear][:n]
+    n = x.shape[0]
+    ff_part = _part(FEED_FORWARDS, "clamped_experts", {"hidden_size": H, "experts": E, "top": top, "ff": ff, "limit": 1.5,
+                                                       "shared_ff": sff, "shared_limit": 0.8}, w, dtype)
+    got = _sum_terms(ff_part.forward(x.to(DEV)))
+    names = {"l.router": "router", "l.router.b": "router_bias", "l.shared.gate": "shared_gate", "l.shared.up": "shared_up",
+             "l.shared.down": "shared_down"}
+    names.update({f"l.e{e}.{m}": f"{m}_{e}" for e in range(E) for m in ("gate", "up", "down")})
+    pw = {k: w[v].double() for k, v in names.items() if v in w}
+    mlp = {"kind": "moe", "expert": {"ff": ff, "limit": 1.5}, "router": {"experts": E, "top": top}}
+    if sff:
+        mlp["shared"] = {"ff": sff, "limit": 0.8}
+    want = plain.feed_forward(None, mlp, pw, "l.", x.double())
+    _close(got, want, 1e-5 if dtype == torch.float32 else 2.5e-2, "clamped experts")

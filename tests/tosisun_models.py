@@ -36,7 +36,7 @@ MAIN = dict(
              mlp=dict(kind="dense", ff=136), weights_of=0),
         dict(type="attention",
              mixer=dict(heads=8, kv_heads=2, dim=64, vdim=64, conv=3, scale=0.11,
-                        rot=dict(base=500000.0, dims=32, scaling=dict(factor=4.0, low=1.0, high=4.0, original=32))),
+                        rot=dict(base=1000000.0, dims=32, scaling=dict(factor=4.0, low=1.0, high=4.0, original=32))),
              mlp=dict(kind="moe", expert=dict(ff=24, limit=3.0), router=dict(experts=5, top=1))),
     ])
 
@@ -152,7 +152,7 @@ def random_config(seed):
     cfg = dict(architecture="Tosisun", width=width, vocab=rng.choice([97, 256, 411]),
                norm=dict(eps=rng.choice([1e-6, 1e-5, 3e-6])), layers=[])
     if rng.random() < 0.7:
-        cfg["logit_softcap"] = rng.choice([5.0, 15.0, 40.0])
+        cfg["logit_softcap"] = rng.choice([5.0, 12.0, 40.0])
     owners = []
     for i in range(rng.randint(2, 6)):
         if owners and rng.random() < 0.35:
@@ -164,10 +164,10 @@ def random_config(seed):
         kvh = rng.choice([1, 2, 3, 4])
         dim = rng.choice([8, 16, 24, 32, 48, 64, 96, 128])
         dims = rng.choice([0, 2, dim // 2, dim]) // 2 * 2
-        rot = dict(base=rng.choice([50.0, 10000.0, 500000.0]), dims=dims)
+        rot = dict(base=rng.choice([50.0, 10000.0, 1000000.0]), dims=dims)
         if dims and rng.random() < 0.6:
             rot["scaling"] = dict(factor=rng.choice([2.0, 4.0, 8.0]), low=1.0, high=rng.choice([2.0, 4.0]),
-                                  original=rng.choice([16, 64, 512]))
+                                  original=rng.choice([16, 64, 256]))
         mixer = dict(heads=kvh * rng.choice([1, 2, 4, 6]), kv_heads=kvh, dim=dim, vdim=rng.choice([8, 16, 24, 40, 64, 128]),
                      conv=rng.choice([1, 2, 3, 4, 6]), scale=rng.choice([0.05, 0.1, 0.2]) * (32.0 / dim) ** 0.5, rot=rot)
         r = rng.random()
