@@ -23,7 +23,8 @@ def _close(got, want, tol, what=""):
 
 
 # ---- layer norm -----------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("n, H", [(1, 40), (3, 96), (70, 200), (130, 1024), (5, 4100), (66, 1100)])
+@pytest.mark.parametrize("n, H", [(1, 40), (3, 96), (70, 200), (130, 1024), (5, 4100), (66, 1100), (2, 50), (70, 1030), (5, 4098),
+                                  (3, 8200)])
 def test_layer_norm_alone_and_on_a_sublayers_output(n, H):
     g = torch.Generator().manual_seed(n * 1000 + H)
     x = torch.randn(n, H, generator=g) * 3 + 0.7
