@@ -66,6 +66,13 @@ def test_weights_of_may_lead_over_another_such_layer_and_to_a_later_one():
     assert "l4.mix.q" in expected_weights(fc) and "l0.mix.q" not in expected_weights(fc)
 
 
+def test_a_layer_with_anothers_weights_is_described_by_its_owner():
+    cfg = copy.deepcopy(models.MAIN)
+    del cfg["layers"][2]["mlp"]                       # what such an entry repeats of its owner's is not read
+    fc = tosisun_forward_config(TosisunConfig.from_dict(cfg))
+    assert fc.schedule[2].layer == fc.schedule[1].layer == 1
+
+
 def _broken(change):
     cfg = copy.deepcopy(models.MAIN)
     change(cfg)
@@ -84,7 +91,6 @@ def _broken(change):
     (lambda c: c["layers"][2].update(weights_of=2), "weights_of"),
     (lambda c: c["layers"][4].update(weights_of=9), "weights_of"),
     (lambda c: (c["layers"][1].update(weights_of=2), c["layers"][2].update(weights_of=1)), "weights_of"),
-    (lambda c: c["layers"][2]["mixer"].update(dim=32), "weights"),
     (lambda c: c["layers"][1]["mlp"]["router"].update(top=7), "top"),
     (lambda c: c["layers"][1]["mlp"]["expert"].pop("limit"), "limit"),
     (lambda c: c["layers"][1]["mlp"]["shared"].pop("limit"), "shared"),

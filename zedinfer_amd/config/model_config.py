@@ -325,15 +325,14 @@ class TosisunConfig(ModelConfig):
         if self.logit_softcap < 0:
             raise ConfigError(f"config.json: logit_softcap must be positive, got {self.logit_softcap}")
         for i, layer in enumerate(self.layers):
+            if isinstance(layer, Mapping) and layer.get("weights_of") is not None:
+                # such a layer is its owner's parts once more: what else its entry says repeats the owner's entry and
+                # is not read
+                self.owner_of(i)
+                continue
             kind = layer.get("type") if isinstance(layer, Mapping) else None
             if kind not in self.MIXER_KEYS:
                 raise ConfigError(f"config.json: layer {i} has type {kind!r}; known: {', '.join(sorted(self.MIXER_KEYS))}")
-            if layer.get("weights_of") is not None:
-                src = self.owner_of(i)
-                o = self.layers[src]
-                if (o.get("type"), o.get("mixer"), o.get("mlp")) != (layer.get("type"), layer.get("mixer"), layer.get("mlp")):
-                    raise ConfigError(f"config.json: layer {i}: a layer that uses layer {src}'s weights must equal it in "
-                                      "type, mixer and mlp")
             m = layer.get("mixer")
             lacking = [k for k in self.MIXER_KEYS[kind] if not isinstance(m, Mapping) or k not in m]
             if lacking:

@@ -85,7 +85,7 @@ def tosisun_forward_config(cfg: TosisunConfig) -> ModelForwardConfig:
         lm_head=PartSpec("linear", {"vocab_size": cfg.vocab_size, "hidden_size": H, "tied_to": None,
                                     "softcap": cfg.logit_softcap or None}, {"weight": "head"}),
         eos_token_ids=cfg.eos_token_ids, max_position_embeddings=0,
-        family={"mixers": [layer["type"] for layer in cfg.layers], "norm_eps": cfg.norm_eps})
+        family={"mixers": [cfg.layers[cfg.owner_of(i)]["type"] for i in range(len(cfg.layers))], "norm_eps": cfg.norm_eps})
     fc.validate()
     return fc
 
